@@ -196,8 +196,9 @@ __global__ __launch_bounds__(kAttnThreads) void sparse_decode_kernel(
   // The partials cross workgroups inside one launch.  They are written and read with agent-scope
   // relaxed atomics (write-through stores, cache-bypassing loads) instead of plain accesses fenced
   // by __threadfence(): an agent-scope fence on this multi-die part writes back and invalidates a
-  // whole L2, once per workgroup.  The barrier below makes every wave wait for its own stores
-  // before thread 0 bumps the arrival counter.
+  // whole L2, once per workgroup.  Every storing wave waits for the acknowledgement of its own
+  // write-through stores (the barrier alone waits for LDS traffic only), then the barrier orders
+  // all of them ahead of the arrival counter that thread 0 bumps.
   if (tid < kHeadDim) {
     if (tid == 0) {
       __hip_atomic_store(mine + 0, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -205,6 +206,7 @@ __global__ __launch_bounds__(kAttnThreads) void sparse_decode_kernel(
     }
     __hip_atomic_store(mine + 2 + tid, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  wait_own_stores();
   __syncthreads();
   if (tid == 0) {
     const uint32_t prev = atomicAdd(&counters[bh], 1u);
@@ -356,6 +358,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_kernel(
   float* mine = partial + (bh * kMaxSplits + split) * kPartialFloats;
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
+  wait_own_stores();
   __syncthreads();
   uint32_t* counter = counters + static_cast<size_t>(b) * num_heads + hg * kDenseHeads;
   if (tid == 0) {
@@ -530,6 +533,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_kernel(
   float* mine = partial + (bh * kMaxSplits + split) * kPartialFloats;
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
+  wait_own_stores();
   __syncthreads();
   uint32_t* counter = counters + static_cast<size_t>(b) * num_heads + head0;
   if (tid == 0) {

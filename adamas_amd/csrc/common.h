@@ -26,6 +26,13 @@ __device__ __forceinline__ int wave_id_uniform() {
   return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
 }
 
+// Waits until every global store this wave has issued is acknowledged by the memory system.  A
+// workgroup barrier does not: it waits for LDS traffic only, so a wave that publishes data with
+// write-through stores for another workgroup calls this before the barrier that precedes the flag.
+__device__ __forceinline__ void wait_own_stores() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 __device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) & 63; }
 
 // 4-level bucket of a Hadamard output value: (v > -10) + (v > 0) + (v > 10).

@@ -426,7 +426,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   int32_t* sdst = sel_out ? sel_out + static_cast<size_t>(bh) * k : nullptr;
   if (!kFromQkv && tid == 0) sh.rows[n_take] = cur_row;  // the current token closes the list
   __syncthreads();
-  // the selection goes out after the barrier: a barrier waits for outstanding global stores
+  // the selection goes out once the row list is complete (every wave has emitted its part)
   if (sdst)
     for (uint32_t i = tid; i < k; i += kAttThreads) sdst[i] = i < n_take ? sh.sel_pos[i] : -1;
   if (kFromQkv) {

@@ -29,6 +29,7 @@ __all__ = [
     "PagePool",
     "PagedSequences",
     "InferenceController",
+    "BatchDecodeWithPagedKVCacheWrapper",
     "ALL_PAST_TOKENS",
     "hadamard_transform",
     "pack_2bit",
@@ -202,14 +203,22 @@ def decode_estimate(q: torch.Tensor, iController: InferenceController, layer_idx
     out = buf[:, :, :lmax - 1]
     if c.batch_size == 1:
         out = out[0]
-    out._adamas_integer_distance = True  # lets decode_topk take the single-pass integer select
+    # the controller remembers the buffer it handed out: decode_topk takes the single-pass integer
+    # selection for any view of it (slices, reshapes), whatever the caller did to the tensor object
+    c._estimate_storage = (buf.untyped_storage().data_ptr(), buf.untyped_storage().nbytes())
     return out
 
 
-def decode_topk(estimated_attn_score: torch.Tensor, iController: InferenceController):
+def decode_topk(estimated_attn_score: torch.Tensor, iController: InferenceController,
+                integer_keys: Optional[bool] = None):
     """Select the budget-1 past tokens with the SMALLEST estimate per head, ties to the lowest index.
     Fills iController.topk_dindices_buffer (logical token positions, int32) and topk_dout_buffer
     (their estimates).  Reference: adamas/utils/__init__.py:239-269.
+
+    integer_keys: True promises that every estimate is an integer in [0, 511] (what decode_estimate
+    produces) and selects with one histogram pass; False takes the selection for arbitrary fp16
+    keys.  None (the reference's two-argument call) decides by whether the tensor is a view of the
+    buffer the controller's last decode_estimate filled; a copy of it is treated as arbitrary keys.
     """
     c = iController
     est = estimated_attn_score
@@ -231,7 +240,10 @@ def decode_topk(estimated_attn_score: torch.Tensor, iController: InferenceContro
     if n < k and c.batch_size == 1:
         # reference check CHECK_GE(num_pages, page_budget) in adamas/ops/csrc/topk.cu:26
         raise RuntimeError("fewer candidates than the budget")
-    mode = _lib.KEY_FP16_INT if getattr(est, "_adamas_integer_distance", False) else _lib.KEY_FP16_GENERIC
+    if integer_keys is None:
+        base, nbytes = getattr(c, "_estimate_storage", (0, 0))
+        integer_keys = nbytes > 0 and base <= est.data_ptr() < base + nbytes
+    mode = _lib.KEY_FP16_INT if integer_keys else _lib.KEY_FP16_GENERIC
     ragged = c.batch_size > 1
     buf = c.topk_workspace(n, k)
     rc = _lib.load().adamas_topk(est2.data_ptr(), est2.stride(0), n,
@@ -274,6 +286,106 @@ def decode_sparse_attn(q: torch.Tensor, iController: InferenceController, layer_
         _lib.current_stream())
     _lib.check(rc, "adamas_sparse_decode")
     return o
+
+
+class BatchDecodeWithPagedKVCacheWrapper:
+    """Counterpart of the reference's decode wrapper (adamas/utils/decode_wrapper.py:11-82; exported by
+    adamas/utils/__init__.py:9,15): attention of one new token over a per-head list of physical
+    pages plus the (partly filled) last page, with the reference's method names and argument lists.
+
+    The reference plans split-KV work and allocates temporary buffers in begin_forward
+    (decode_handler.cuh:73-136); the HIP kernel splits and merges on its own, so begin_forward only
+    records the sizes and end_forward has nothing to free.  forward() maps the page list onto
+    adamas_sparse_decode: the pool's pages in identity order form a virtual sequence whose one extra
+    page is `paged_kv_last_page_idx`, every slot of a listed page becomes a token position of that
+    sequence, and the newest token is the last valid slot of the extra page.  One sequence, as in
+    the reference (batch_size 1, approx_attn.cu:78).  decode_sparse_attn is the path the model
+    takes; this class serves callers that hold page lists of their own."""
+
+    def __init__(self, kv_layout: str = "NHD"):
+        if not hasattr(TensorLayout, kv_layout) or kv_layout not in ("NHD", "HND"):
+            raise KeyError("Invalide kv_layout {}".format(kv_layout))  # (sic) the reference's message
+        self.kv_layout = kv_layout
+        self._plan = None
+        self._table = None
+        self._workspace = None
+
+    def begin_forward(self, indptr: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
+                      head_dim: int, page_size: int, data_type):
+        """indptr = [0, pages listed per head] (one sequence).  Reads indptr once, here."""
+        if head_dim != 128:
+            raise RuntimeError("BatchDecodeWithPagedKVCacheWrapper supports head_dim 128 only")
+        if num_qo_heads % num_kv_heads != 0:
+            raise RuntimeError("num_qo_heads must be a multiple of num_kv_heads")
+        if data_type not in _FLOAT_DTYPES:
+            raise RuntimeError("BatchDecodeWithPagedKVCacheWrapper failed to dispatch with dtype %s"
+                               % data_type)
+        if indptr.numel() != 2:
+            raise RuntimeError("indptr must be [0, n_pages] of one sequence")
+        n_listed = int(indptr.reshape(-1)[1].item()) - int(indptr.reshape(-1)[0].item())
+        if n_listed < 0:
+            raise RuntimeError("indptr must not decrease")
+        self._plan = (n_listed, num_qo_heads, num_kv_heads, page_size, data_type)
+
+    def end_forward(self):
+        self._plan = None
+
+    def forward(self, q: torch.Tensor, o: torch.Tensor, paged_kv_data: torch.Tensor,
+                paged_kv_indices: torch.Tensor, paged_kv_indptr: torch.Tensor,
+                paged_kv_last_page_len: int, paged_kv_last_page_idx: int,
+                rope_scale: Optional[float] = None, rope_theta: Optional[float] = None):
+        """q, o [1, Hq, 128]; paged_kv_data [pages, 2, P, Hkv, 128] (NHD) or [pages, 2, Hkv, P, 128];
+        paged_kv_indices [Hq, row stride] int32 physical page ids, the first indptr[1] of every row
+        are attended in full; the first paged_kv_last_page_len slots of page paged_kv_last_page_idx
+        are attended too (its last valid slot is the newest token).  rope_* are accepted and unused
+        (RotaryMode::kNone in the reference, approx_attn.cu:135).  Writes o."""
+        if self._plan is None:
+            # the reference's handler throws when forward comes before begin_forward
+            # (decode_handler.cuh:226-231)
+            raise RuntimeError("BatchDecodeWithPagedKVCacheWrapper: begin_forward must come first")
+        n_listed, nq, nkv, page, dtype = self._plan
+        _check_cuda_contig(q, "q", dtype, 3)
+        _check_cuda_contig(o, "o", dtype, 3)
+        _check_cuda_contig(paged_kv_data, "paged_kv_data", dtype, 5)
+        _check_cuda_contig(paged_kv_indices, "paged_kv_indices", torch.int32, 2)
+        hnd = self.kv_layout == "HND"
+        want = (2, nkv, page, 128) if hnd else (2, page, nkv, 128)
+        if tuple(paged_kv_data.shape[1:]) != want:
+            raise RuntimeError("paged_kv_data must be [pages, %s]" % ", ".join(map(str, want)))
+        if q.shape != (1, nq, 128) or o.shape != q.shape:
+            raise RuntimeError("q and o must be [1, num_qo_heads, 128]")
+        if paged_kv_indices.shape[0] != nq or paged_kv_indices.shape[1] < n_listed:
+            raise RuntimeError("paged_kv_indices must be [num_qo_heads, >= indptr[1]]")
+        n_pool = paged_kv_data.shape[0]
+        last_len, last_idx = int(paged_kv_last_page_len), int(paged_kv_last_page_idx)
+        if not (1 <= last_len <= page and 0 <= last_idx < n_pool):
+            raise RuntimeError("last page: 1 <= len <= page_size and a valid page id expected")
+        dev = q.device
+        if self._table is None or self._table.numel() != n_pool + 1 or self._table.device != dev:
+            self._table = torch.arange(n_pool + 1, dtype=torch.int32, device=dev)
+            self._indptr = torch.tensor([0, n_pool + 1], dtype=torch.int32, device=dev)
+            self._len = torch.zeros(1, dtype=torch.int32, device=dev)
+        self._table[n_pool] = last_idx
+        seq_len = n_pool * page + last_len
+        self._len.fill_(seq_len)
+        slots = torch.arange(page, dtype=torch.int32, device=dev)
+        pos = (paged_kv_indices[:, :n_listed, None] * page + slots).reshape(nq, n_listed * page)
+        tail = (n_pool * page + slots[:last_len - 1]).expand(nq, last_len - 1)
+        sel = torch.cat((pos, tail), dim=1).contiguous()
+        if sel.shape[1] == 0:   # only the newest token: one unused entry (a null list means "dense")
+            sel = torch.full((nq, 1), -1, dtype=torch.int32, device=dev)
+        n_sel = sel.shape[1]
+        lib = _lib.load()
+        need = lib.adamas_workspace_bytes(1, nq, 1, 1)
+        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != dev:
+            self._workspace = torch.zeros(need, dtype=torch.uint8, device=dev)
+        flags = _lib.dtype_flags(dtype) | (_lib.F_HND if hnd else 0)
+        rc = lib.adamas_sparse_decode_f(
+            q.data_ptr(), paged_kv_data.data_ptr(), self._table.data_ptr(), self._indptr.data_ptr(),
+            self._len.data_ptr(), sel.data_ptr(), max(n_sel, 1), n_sel, o.data_ptr(),
+            self._workspace.data_ptr(), self._workspace.numel(), 1, nq, nkv, 128, page,
+            1.0 / math.sqrt(128), seq_len, flags, _lib.current_stream())
+        _lib.check(rc, "adamas_sparse_decode")
 
 
 def decode_step(q: torch.Tensor, q_code: torch.Tensor, iController: InferenceController,

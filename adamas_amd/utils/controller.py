@@ -91,7 +91,7 @@ class InferenceController:
 
         # workspace of the attention kernel and of the fused step (zero-filled once)
         self._workspace: Optional[torch.Tensor] = None
-        self._workspace_budget = -1
+        self._workspace_need = {}
         self._len_bound: Optional[int] = None
 
     # --- device-side views used by the operator functions -----------------------------------------
@@ -120,12 +120,20 @@ class InferenceController:
         return min(self.seqs.lengths)
 
     def workspace(self, budget: int) -> torch.Tensor:
+        """Workspace of the attention kernel and of the step for this token budget.  The size the
+        library asks for is not monotonic in the budget (different budgets take different paths),
+        so reuse is decided by bytes; a budget that keeps growing (dense layers: budget = length)
+        is sized for the next power of two, which bounds the number of reallocations."""
         budget = max(1, min(int(budget), self.max_seq_len))
-        if self._workspace is None or budget > self._workspace_budget:
-            nbytes = _lib.load().adamas_workspace_bytes(self.batch_size, self.num_heads,
-                                                        self.max_seq_len, budget)
-            self._workspace = torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
-            self._workspace_budget = budget
+        need = self._workspace_need.get(budget)
+        if need is None:
+            fn = _lib.load().adamas_workspace_bytes
+            ahead = min(self.max_seq_len, 1 << (budget - 1).bit_length())
+            need = max(fn(self.batch_size, self.num_heads, self.max_seq_len, budget),
+                       fn(self.batch_size, self.num_heads, self.max_seq_len, ahead))
+            self._workspace_need[budget] = need
+        if self._workspace is None or need > self._workspace.numel():
+            self._workspace = torch.zeros(need, dtype=torch.uint8, device=self.device)
         return self._workspace
 
     def topk_workspace(self, n: int, k: int) -> torch.Tensor:

@@ -109,6 +109,20 @@ def test_workspace_bytes_grows_with_sizes():
     assert a % 256 == 0
 
 
+def test_controller_workspace_covers_a_lowered_budget():
+    """The size the library asks for is not monotonic in the budget: a controller that has served
+    budget 300 must still hand out enough bytes for 256 (and a growing dense budget must not
+    reallocate at every token)."""
+    lib = _lib.load()
+    c = _ctrl(max_seq_len=32768, num_layers=1)
+    for budget in (300, 256, 200, 128, 4096, 129):
+        ws = c.workspace(budget)
+        assert ws.numel() >= lib.adamas_workspace_bytes(1, 32, 32768, budget), budget
+    c = _ctrl(max_seq_len=32768, num_layers=1)
+    seen = {c.workspace(b).data_ptr() for b in range(20000, 20600)}
+    assert len(seen) == 1
+
+
 def _ctrl(**kw):
     args = dict(num_layers=2, num_heads=32, head_dim=128, page_size=16, page_budget=64,
                 max_seq_len=256, dtype=torch.float16, device="cpu")

@@ -324,9 +324,12 @@ def test_sparse_attention_one_hot_v_and_padding(gpu_device):
 
 
 # ------------------------------------------------------------------------------ whole step ------
-def _run_step(gpu_device, seq, budget, page_size, shuffle_seed, fused_append=True):
+SCALES = [1.0, 128 ** -0.5]   # raw butterfly (this build's default) and the orthonormal transform
+
+
+def _run_step(gpu_device, seq, budget, page_size, shuffle_seed, fused_append=True, scale=1.0):
     L = seq.k.shape[0]
-    ctrl = T.make_controller(gpu_device, L, budget, page_size, shuffle_seed=shuffle_seed)
+    ctrl = T.make_controller(gpu_device, L, budget, page_size, shuffle_seed=shuffle_seed, scale=scale)
     k, v, q = seq.k.to(gpu_device), seq.v.to(gpu_device), seq.q.to(gpu_device)
     T.fill_sequence(ctrl, k[:L - 1], v[:L - 1])
     q_code = T.decode_append(ctrl, q[None], k[L - 1:], v[L - 1:], fused=fused_append)
@@ -339,9 +342,9 @@ def _run_step(gpu_device, seq, budget, page_size, shuffle_seed, fused_append=Tru
     return ctrl, q_code, est, sel, o, o_fused, sel_fused.clone()
 
 
-def _check_step(seq, budget, q_code, est, sel, o, o_fused, sel_fused):
+def _check_step(seq, budget, q_code, est, sel, o, o_fused, sel_fused, scale=1.0):
     L = seq.k.shape[0]
-    ora = T.oracle_step(seq.q, seq.k, seq.v, budget)
+    ora = T.oracle_step(seq.q, seq.k, seq.v, budget, scale=scale)
     assert np.array_equal(T.words_u16(q_code)[0], ora["q_words"])
     assert np.array_equal(T.np16(est).astype(np.int32), ora["dist"])
     ok, h = T.sets_equal(T.np16(sel), ora["sets"], L)
@@ -353,14 +356,22 @@ def _check_step(seq, budget, q_code, est, sel, o, o_fused, sel_fused):
     return ora
 
 
-def test_step_config1_4k_budget64(gpu_device):
+# The scale of the reference's third-party Hadamard transform is not fixed by anything in its tree,
+# so every configuration runs at both candidates.  With the orthonormal scale the synthetic inputs
+# give codes 1 and 2 almost everywhere, distances fall into a few bins and most of a selection is
+# decided by the lowest-index tie rule: the tie quota paths of both selection levels at full size.
+@pytest.mark.parametrize("scale", SCALES)
+def test_step_config1_4k_budget64(gpu_device, scale):
     w = synth.WORKLOADS["c1_4k_b64"]
     seq = synth.make_workload(w)[0]
-    _, q_code, est, sel, o, o_f, sel_f = _run_step(gpu_device, seq, w.budget, w.page_size, 1)
-    ora = _check_step(seq, w.budget, q_code, est, sel, o, o_f, sel_f)
-    # the planted needles are among the selected tokens
-    for h in range(32):
-        assert set(seq.needles[h].tolist()) <= set(int(x) for x in ora["sets"][h])
+    _, q_code, est, sel, o, o_f, sel_f = _run_step(gpu_device, seq, w.budget, w.page_size, 1,
+                                                   scale=scale)
+    ora = _check_step(seq, w.budget, q_code, est, sel, o, o_f, sel_f, scale=scale)
+    if scale == 1.0:
+        # the planted needles are among the selected tokens (with the orthonormal scale the codes
+        # are too coarse to tell them apart from their many ties)
+        for h in range(32):
+            assert set(seq.needles[h].tolist()) <= set(int(x) for x in ora["sets"][h])
 
 
 def test_step_config1_page_size_1_unfused(gpu_device):
@@ -371,23 +382,27 @@ def test_step_config1_page_size_1_unfused(gpu_device):
 
 
 @pytest.mark.timeout(600)
-def test_step_config2_32k_budget128(gpu_device):
+@pytest.mark.parametrize("scale", SCALES)
+def test_step_config2_32k_budget128(gpu_device, scale):
     w = synth.WORKLOADS["c2_32k_b128"]
     T.heartbeat("config 2: generating inputs")
     seq = synth.make_workload(w)[0]
     T.heartbeat("config 2: running the HIP path")
-    _, q_code, est, sel, o, o_f, sel_f = _run_step(gpu_device, seq, w.budget, w.page_size, 2)
-    _check_step(seq, w.budget, q_code, est, sel, o, o_f, sel_f)
+    _, q_code, est, sel, o, o_f, sel_f = _run_step(gpu_device, seq, w.budget, w.page_size, 2,
+                                                   scale=scale)
+    _check_step(seq, w.budget, q_code, est, sel, o, o_f, sel_f, scale=scale)
 
 
 @pytest.mark.timeout(900)
-def test_step_config4_128k_budget256(gpu_device):
+@pytest.mark.parametrize("scale", SCALES)
+def test_step_config4_128k_budget256(gpu_device, scale):
     w = synth.WORKLOADS["c4_128k_b256"]
     T.heartbeat("config 4: generating inputs")
     seq = synth.make_workload(w)[0]
     T.heartbeat("config 4: running the HIP path")
-    _, q_code, est, sel, o, o_f, sel_f = _run_step(gpu_device, seq, w.budget, w.page_size, 4)
-    _check_step(seq, w.budget, q_code, est, sel, o, o_f, sel_f)
+    _, q_code, est, sel, o, o_f, sel_f = _run_step(gpu_device, seq, w.budget, w.page_size, 4,
+                                                   scale=scale)
+    _check_step(seq, w.budget, q_code, est, sel, o, o_f, sel_f, scale=scale)
 
 
 @pytest.mark.timeout(900)
@@ -519,7 +534,8 @@ def test_step_wide_distance_spread(gpu_device):
     assert np.abs(T.np16(o_f)[0].astype(np.float64) - ora["out"]).max() <= 2e-2
 
 
-def test_step_ragged_batch(gpu_device):
+@pytest.mark.parametrize("scale", SCALES)
+def test_step_ragged_batch(gpu_device, scale):
     """Batched ragged decode (no reference implementation: the oracle is the single-sequence oracle
     applied per sequence).  Lengths are scaled down so the oracle finishes in seconds; one sequence
     is shorter than the budget and must fall back to attending everything."""
@@ -528,7 +544,7 @@ def test_step_ragged_batch(gpu_device):
     g = torch.Generator().manual_seed(3)
     seqs = [synth.make_sequence(L, 8, g) for L in lens]
     B = len(lens)
-    ctrl = T.make_controller(gpu_device, 3072, budget, 16, batch_size=B, shuffle_seed=3)
+    ctrl = T.make_controller(gpu_device, 3072, budget, 16, batch_size=B, shuffle_seed=3, scale=scale)
     for b, s in enumerate(seqs):
         T.fill_sequence(ctrl, s.k[:-1].to(gpu_device), s.v[:-1].to(gpu_device), seq_idx=b)
     q = torch.stack([s.q for s in seqs]).to(gpu_device)
@@ -542,7 +558,7 @@ def test_step_ragged_batch(gpu_device):
     o_f, sel_f = U.decode_step(q, q_code, ctrl, 0, return_indices=True)
     for b, s in enumerate(seqs):
         L = lens[b]
-        ora = T.oracle_step(s.q, s.k, s.v, budget)
+        ora = T.oracle_step(s.q, s.k, s.v, budget, scale=scale)
         assert np.array_equal(T.words_u16(q_code)[b], ora["q_words"])
         assert np.array_equal(T.np16(est[b, :, :L - 1]).astype(np.int32), ora["dist"])
         for which in (sel, sel_f):
