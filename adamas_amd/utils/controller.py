@@ -119,21 +119,29 @@ class InferenceController:
     def min_len_now(self) -> int:
         return min(self.seqs.lengths)
 
-    def workspace(self, budget: int) -> torch.Tensor:
-        """Workspace of the attention kernel and of the step for this token budget.  The size the
-        library asks for is not monotonic in the budget (different budgets take different paths),
-        so reuse is decided by bytes; a budget that keeps growing (dense layers: budget = length)
-        is sized for the next power of two, which bounds the number of reallocations."""
+    def workspace(self, budget: int, max_len: Optional[int] = None) -> torch.Tensor:
+        """Workspace of the attention kernel and of the step for this token budget and the length
+        bound the library is called with (`max_len`, by default max_len_now, which is what the
+        operator functions pass).  The size the library asks for is monotonic neither in the budget
+        nor in the length (different sizes take different paths), so reuse is decided by bytes, for
+        exactly the sizes of the call; a new buffer is sized with a quarter of slack and for the
+        full capacity too, so that a sequence growing token by token (or a dense budget that grows
+        with it) reallocates a bounded number of times."""
         budget = max(1, min(int(budget), self.max_seq_len))
-        need = self._workspace_need.get(budget)
+        max_len = self.max_len_now if max_len is None else int(max_len)
+        max_len = max(1, min(max_len, self.max_seq_len))
+        key = (budget, max_len)
+        need = self._workspace_need.get(key)
         if need is None:
-            fn = _lib.load().adamas_workspace_bytes
-            ahead = min(self.max_seq_len, 1 << (budget - 1).bit_length())
-            need = max(fn(self.batch_size, self.num_heads, self.max_seq_len, budget),
-                       fn(self.batch_size, self.num_heads, self.max_seq_len, ahead))
-            self._workspace_need[budget] = need
+            need = _lib.load().adamas_workspace_bytes(self.batch_size, self.num_heads, max_len, budget)
+            if len(self._workspace_need) > 4096:
+                self._workspace_need.clear()
+            self._workspace_need[key] = need
         if self._workspace is None or need > self._workspace.numel():
-            self._workspace = torch.zeros(need, dtype=torch.uint8, device=self.device)
+            full = _lib.load().adamas_workspace_bytes(self.batch_size, self.num_heads,
+                                                      self.max_seq_len, budget)
+            size = (max(need, full) * 5 // 4 + 255) // 256 * 256
+            self._workspace = torch.zeros(size, dtype=torch.uint8, device=self.device)
         return self._workspace
 
     def topk_workspace(self, n: int, k: int) -> torch.Tensor:

@@ -109,18 +109,27 @@ def test_workspace_bytes_grows_with_sizes():
     assert a % 256 == 0
 
 
-def test_controller_workspace_covers_a_lowered_budget():
-    """The size the library asks for is not monotonic in the budget: a controller that has served
-    budget 300 must still hand out enough bytes for 256 (and a growing dense budget must not
-    reallocate at every token)."""
+def test_controller_workspace_covers_every_size_it_is_asked_for():
+    """The size the library asks for is monotonic neither in the budget nor in the length: a
+    controller that has served one size must still hand out enough bytes for the next, whatever
+    the order (budget 300 then 256; 32832 tokens then 32769), and a sequence or a dense budget that
+    grows token by token must not reallocate at every token."""
     lib = _lib.load()
-    c = _ctrl(max_seq_len=32768, num_layers=1)
-    for budget in (300, 256, 200, 128, 4096, 129):
+    assert lib.adamas_workspace_bytes(1, 32, 32769, 128) > lib.adamas_workspace_bytes(1, 32, 32832, 128)
+    c = _ctrl(max_seq_len=32832, num_layers=1)
+    c.prepare_hadamard(32769)
+    for budget in (32769, 128, 300, 256, 200, 128, 4096, 129):
         ws = c.workspace(budget)
-        assert ws.numel() >= lib.adamas_workspace_bytes(1, 32, 32768, budget), budget
-    c = _ctrl(max_seq_len=32768, num_layers=1)
-    seen = {c.workspace(b).data_ptr() for b in range(20000, 20600)}
-    assert len(seen) == 1
+        assert ws.numel() >= lib.adamas_workspace_bytes(1, 32, 32769, budget), budget
+    seen = set()
+    for _ in range(40):
+        c.prepare_hadamard(1)
+        n = c.max_len_now
+        for budget in (n, 128):       # the dense layers, then the sparse ones, as a model alternates
+            ws = c.workspace(budget)
+            assert ws.numel() >= lib.adamas_workspace_bytes(1, 32, n, budget)
+            seen.add(ws.data_ptr())
+    assert len(seen) <= 2
 
 
 def _ctrl(**kw):
