@@ -42,6 +42,10 @@ _SIGNATURES = {
                                     c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float,
                                     c_uint32, c_uint32, c_void_p]),
     "adamas_step_fused_supported": (c_int, [c_uint32, c_uint32, c_uint32, c_uint32]),
+    "adamas_decode_step_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32,
+                                            c_uint32, c_uint32, c_uint32, c_float, c_uint32, c_uint32,
+                                            c_uint32, c_void_p]),
     "adamas_step_candidates": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32,
                                         c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32,
                                         c_uint32, c_uint32, c_void_p]),
@@ -87,6 +91,8 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 F_CODE_FROM_FP32 = 1
 F_BF16 = 2
 F_HND = 4
+STATIC_SCRATCH_BYTES = 24 << 20
+E_SCRATCH = -5
 DIST_FP16, DIST_U16 = 0, 1
 KEY_FP16_GENERIC, KEY_FP16_INT, KEY_U16_INT = 0, 1, 2
 

@@ -754,6 +754,7 @@ extern "C" const char* adamas_error_string(int code) {
     case ADAMAS_E_UNSUPPORTED: return "adamas: unsupported shape (head_dim must be 128, num_heads a multiple of 32)";
     case ADAMAS_E_WORKSPACE: return "adamas: workspace missing or too small";
     case ADAMAS_E_ALIGN: return "adamas: pointer or stride not aligned as documented";
+    case ADAMAS_E_SCRATCH: return "adamas: sizes beyond the static scratch (ADAMAS_STATIC_SCRATCH_BYTES) of adamas_decode_step_noalloc";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));

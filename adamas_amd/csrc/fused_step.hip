@@ -885,3 +885,55 @@ extern "C" int adamas_decode_layer_step(const void* qkv, const float* cos_table,
                           head_dim, page_size, sm_scale, max_seq_len, page_table_stride, 0u, stream,
                           &src, code_data);
 }
+
+// ---- the decode step for callers that cannot allocate ----------------------------------------------
+// The workspace of adamas_decode_step_f lives in a file-scope device array instead of caller memory:
+// every GPU the library runs on holds one copy of it (ADAMAS_STATIC_SCRATCH_BYTES) until the process
+// ends.  In host code the array's name is only a handle: its device address is asked for once per
+// device (hipGetSymbolAddress, with that device current) and kept; kernels receive that address as
+// the workspace pointer, exactly as they receive a caller's buffer.  The array is zero at load, which
+// is the state the split-merge arrival counters need; every kernel that uses a counter puts it back
+// to zero, and candidates, histograms and partial sums are written before they are read within one
+// call, so a call finds what it needs whatever the previous call (of any size) left behind.  Calls
+// that overlap on one GPU (two streams, two threads) share the array and race.
+static __device__ __align__(256) unsigned char scratch[ADAMAS_STATIC_SCRATCH_BYTES];
+
+static int static_scratch_address(void** out) {
+  static std::atomic<void*> per_device[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= 64) return ADAMAS_E_UNSUPPORTED;
+  void* p = per_device[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (!p) return ADAMAS_E_SCRATCH;
+    per_device[dev].store(p, std::memory_order_release);  // every thread finds the same address
+  }
+  *out = p;
+  return 0;
+}
+
+extern "C" int adamas_decode_step_noalloc(const void* q, const void* q_code, const void* kv_data,
+                                          const void* code_data, const int32_t* page_indices,
+                                          const int32_t* page_indptr, const int32_t* seq_lens,
+                                          uint32_t budget, void* out, int32_t* sel_out,
+                                          uint32_t batch, uint32_t num_heads, uint32_t num_kv_heads,
+                                          uint32_t head_dim, uint32_t page_size, float sm_scale,
+                                          uint32_t max_seq_len, uint32_t page_table_stride,
+                                          uint32_t flags, adamas_stream_t stream) {
+  if (budget == 0 || max_seq_len == 0 || batch == 0 || num_heads == 0) return ADAMAS_E_BADARG;
+  // sizes first: the product below must not wrap before it is compared with the limit
+  if (batch > 65535 || num_heads > 65535 || max_seq_len > (1u << 24) || budget > (1u << 24))
+    return ADAMAS_E_SCRATCH;
+  const WorkspaceLayout w = workspace_layout(batch, num_heads, max_seq_len, budget);
+  if (w.total > ADAMAS_STATIC_SCRATCH_BYTES) return ADAMAS_E_SCRATCH;
+  void* ws = nullptr;
+  const int rc = static_scratch_address(&ws);
+  if (rc != 0) return rc;
+  return adamas_decode_step_f(q, q_code, kv_data, code_data, page_indices, page_indptr, seq_lens,
+                              budget, out, sel_out, ws, ADAMAS_STATIC_SCRATCH_BYTES, batch, num_heads,
+                              num_kv_heads, head_dim, page_size, sm_scale, max_seq_len,
+                              page_table_stride, flags, stream);
+}

@@ -48,6 +48,10 @@ typedef void* adamas_stream_t;
 #define ADAMAS_E_UNSUPPORTED (-2) /* head_dim != 128, num_heads not a multiple of 32, ... */
 #define ADAMAS_E_WORKSPACE (-3)   /* workspace too small                                  */
 #define ADAMAS_E_ALIGN (-4)       /* pointer or stride not aligned as documented          */
+#define ADAMAS_E_SCRATCH (-5)     /* sizes beyond the static scratch of adamas_decode_step_noalloc */
+
+/* Bytes of device memory adamas_decode_step_noalloc works in (held by every GPU the library runs on). */
+#define ADAMAS_STATIC_SCRATCH_BYTES (24u << 20)
 
 /* flags for the append / code-generation entry points */
 #define ADAMAS_F_CODE_FROM_FP32 1u /* bucketize the fp32 butterfly output instead of its fp16 rounding */
@@ -252,6 +256,27 @@ int adamas_decode_step_f(const void* q, const void* q_code, const void* kv_data,
                          uint32_t head_dim, uint32_t page_size, float sm_scale,
                          uint32_t max_seq_len, uint32_t page_table_stride, uint32_t flags,
                          adamas_stream_t stream);
+
+/*
+ * adamas_decode_step_f without the workspace arguments, for callers that cannot allocate device
+ * memory (code under HIP graph capture, serving loops and harnesses that forbid it): the library
+ * works in a static device array of ADAMAS_STATIC_SCRATCH_BYTES per GPU instead and calls no
+ * allocating routine.  Sizes whose workspace (adamas_workspace_bytes) exceeds that give
+ * ADAMAS_E_SCRATCH: at 32 heads the limit admits one sequence of up to 131072 tokens at budgets up
+ * to 4096, or two sequences of 32768 tokens at budget 128; larger batches need the caller-workspace
+ * entry point.  All calls on one GPU share the array: calls that overlap on one GPU (different streams
+ * or threads) race; calls on one stream are ordered and fine.  The first call on a device looks up
+ * the array's address (no allocation, but make it outside a stream capture).  Same results as
+ * adamas_decode_step_f, bit for bit.  No counterpart in the reference, whose decode handler
+ * allocates its buffers in every begin_forward (kernels/include/decode/decode_handler.cuh:105-117).
+ */
+int adamas_decode_step_noalloc(const void* q, const void* q_code, const void* kv_data,
+                               const void* code_data, const int32_t* page_indices,
+                               const int32_t* page_indptr, const int32_t* seq_lens, uint32_t budget,
+                               void* out, int32_t* sel_out, uint32_t batch, uint32_t num_heads,
+                               uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size,
+                               float sm_scale, uint32_t max_seq_len, uint32_t page_table_stride,
+                               uint32_t flags, adamas_stream_t stream);
 
 /*
  * The two halves of adamas_decode_step, for callers that want to time or schedule them separately.
