@@ -31,6 +31,7 @@ _SIGNATURES = {
     "adamas_topk": (c_int, [c_void_p, c_int64, c_uint32, c_void_p, c_uint32, c_int32, c_void_p,
                              c_int64, c_uint32, c_uint32, c_void_p, c_void_p, c_int64, c_uint32,
                              c_void_p, c_size_t, c_void_p]),
+    "adamas_read_probe": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "adamas_topk_workspace_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "adamas_workspace_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32, c_uint32]),
     "adamas_sparse_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

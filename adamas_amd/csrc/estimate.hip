@@ -104,9 +104,42 @@ __global__ __launch_bounds__(256) void estimate_kernel(
   }
 }
 
+// Measurement aid: reads `n_vec` 128-bit words and does nothing else (the words are folded into one
+// value that is only stored if it matches a pattern no data holds).  256 workgroups x 512 threads,
+// 16 independent loads in flight per lane, a wave reads 1 KB contiguous per instruction: what the
+// memory system gives a kernel that streams a code cache once, without any of the estimator's work.
+__global__ __launch_bounds__(512) void read_probe_kernel(const uint4* __restrict__ p, uint64_t n_vec,
+                                                         uint32_t* __restrict__ sink) {
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 512u;
+  uint32_t acc = 0;
+  for (uint64_t i0 = static_cast<uint64_t>(blockIdx.x) * 512u + threadIdx.x; i0 < n_vec;
+       i0 += 16 * stride) {
+    uint4 v[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const uint64_t i = i0 + j * stride;
+      v[j] = i < n_vec ? p[i] : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc ^= v[j].x + v[j].y + v[j].z + v[j].w;
+  }
+  if (acc == 0x9e3779b9u && sink) *sink = acc;
+}
+
 }  // namespace adamas
 
 using namespace adamas;
+
+extern "C" int adamas_read_probe(const void* data, size_t bytes, void* sink,
+                                 adamas_stream_t stream) {
+  if (!data || bytes == 0) return ADAMAS_E_BADARG;
+  if ((reinterpret_cast<uintptr_t>(data) & 15) || (bytes & 15)) return ADAMAS_E_ALIGN;
+  hipLaunchKernelGGL(read_probe_kernel, dim3(256), dim3(512), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(data), static_cast<uint64_t>(bytes / 16),
+                     static_cast<uint32_t*>(sink));
+  ADAMAS_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
 
 extern "C" int adamas_estimate(const void* q_code, const void* code_data,
                                const int32_t* page_indices, const int32_t* page_indptr,

@@ -187,6 +187,15 @@ int adamas_topk(const void* values, int64_t row_stride, uint32_t n_max, const in
                 void* out_vals, int64_t out_stride, uint32_t key_mode, void* workspace,
                 size_t workspace_bytes, adamas_stream_t stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: one launch that reads `bytes` bytes at `data`
+ * (16-byte aligned, a multiple of 16) with 128-bit loads, 256 workgroups, 16 loads in flight per
+ * lane, and computes nothing.  Its duration over a code cache is the rate the memory system gives a
+ * kernel that streams those bytes once: the practical ceiling the estimator is compared with.
+ * sink (optional, 4 bytes) is never written for ordinary data.
+ */
+int adamas_read_probe(const void* data, size_t bytes, void* sink, adamas_stream_t stream);
+
 /* Bytes of workspace adamas_topk needs for these sizes (see adamas_topk). */
 size_t adamas_topk_workspace_bytes(uint32_t num_rows, uint32_t n_max, uint32_t k);
 
