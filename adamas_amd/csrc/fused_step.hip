@@ -35,9 +35,14 @@ constexpr int kFusedHeads = 8;                      // the wide workgroup
 constexpr int kAttThreads = 512;
 constexpr int kAttWaves = kAttThreads / kWave;      // 8
 
+// A wave stores the distances of eight heads in one instruction; with rows a multiple of 128 bytes
+// apart those stores would all fall into the same LDS banks, so every row is padded by 16 bytes
+// (eight rows x four words then cover the 32 banks once).
+constexpr uint32_t kDistRowPad = 8;  // u16 elements
+
 template <int kPasses, int kHeads>
 struct EstimateSelectShared {
-  alignas(16) uint16_t dist[kHeads][kFusedBlock * kPasses];  // 0xFFFF = no token
+  alignas(16) uint16_t dist[kHeads][kFusedBlock * kPasses + kDistRowPad];  // 0xFFFF = no token
   uint32_t krow[kFusedBlock * kPasses];       // K row index (page * rows per page + slot) of every token
   // tokens per distance value of one head, two 16-bit bins per word: read off for the chunk's
   // threshold (selection) or written out (histogram mode); rows are read with 128-bit accesses
