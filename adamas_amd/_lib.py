@@ -92,6 +92,7 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 F_CODE_FROM_FP32 = 1
 F_BF16 = 2
 F_HND = 4
+F_NO_MFMA = 8
 STATIC_SCRATCH_BYTES = 24 << 20
 E_SCRATCH = -5
 DIST_FP16, DIST_U16 = 0, 1

@@ -23,7 +23,6 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # packed fp32 instructions are switched off for all device code of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
@@ -36,10 +35,7 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found: set HIPCC or put /opt/rocm/bin on PATH")
 
 
-def build_library(verbose: bool = False) -> Path:
-    """Compile every HIP source into adamas_amd/lib/libadamas_hip.so and return its path."""
-    LIB_DIR.mkdir(parents=True, exist_ok=True)
-    cmd = [find_hipcc(), *HIPCC_FLAGS, *[str(CSRC_DIR / s) for s in SOURCES], "-o", str(LIB_PATH)]
+def _run(cmd, verbose):
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if verbose or proc.returncode != 0:
         print(" ".join(cmd))
@@ -47,6 +43,24 @@ def build_library(verbose: bool = False) -> Path:
         print(proc.stderr)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed with exit code {proc.returncode}")
+
+
+def build_library(verbose: bool = False, jobs: int = 0) -> Path:
+    """Compile every HIP source (one hipcc process each, side by side) and link them into
+    adamas_amd/lib/libadamas_hip.so; returns its path.  Every call recompiles everything."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    LIB_DIR.mkdir(parents=True, exist_ok=True)
+    obj_dir = LIB_DIR / "obj"
+    obj_dir.mkdir(exist_ok=True)
+    hipcc = find_hipcc()
+    jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 8)
+    objects = [obj_dir / (Path(src).stem + ".o") for src in SOURCES]
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(lambda so: _run([hipcc, *HIPCC_FLAGS, "-c", str(CSRC_DIR / so[0]), "-o",
+                                       str(so[1])], verbose), zip(SOURCES, objects)))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *[str(o) for o in objects], "-o",
+          str(LIB_PATH)], verbose)
     return LIB_PATH
 
 

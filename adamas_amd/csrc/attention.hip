@@ -12,10 +12,12 @@
 
 namespace adamas {
 
-constexpr int kAttnThreads = 256;
-constexpr int kGroups = 16;          // rows in flight per load instruction of the workgroup
 constexpr int kTile = 8;             // rows per group per tile
-constexpr int kRowsPerIter = kGroups * kTile;  // 128
+// A workgroup has 256 or 512 threads = 16 or 32 groups, i.e. 128 or 256 rows per tile.  Lists of up to
+// 1024 rows are cut into splits of 128 rows (up to 8 per head: enough workgroups to fill the chip).
+// Longer lists take the wide workgroup and splits of 256 rows: as many rows in flight per CU, half as
+// many partial results to merge, so that up to 4096 rows the merge stays inside the launch.
+constexpr uint32_t kWideRowsFrom = 1025;
 constexpr uint32_t kDeferredMergeSplits = 24;  // splits from which the partials get a merge launch
 // (measured at 32768 tokens, 32 heads: 16 splits 14.7 us merged inside the launch, 15.8 us with a merge
 // launch; 32 splits 26.6 against 22.5 us)
@@ -106,6 +108,7 @@ __device__ __forceinline__ void merge_partial_pairs(const float* base, uint32_t 
   }
 }
 
+template <int kGroups>
 struct AttnShared {
   MergeShared<kGroups> merge;
   uint32_t is_last;
@@ -113,15 +116,16 @@ struct AttnShared {
 
 // kRowIndex: sel_idx holds K row indices (page * 2 * page_size + slot) instead of token positions;
 // only the row of the current token then goes through the page table.
-template <bool kRowIndex, bool kBf16, bool kHnd>
-__global__ __launch_bounds__(kAttnThreads) void sparse_decode_kernel(
+template <bool kRowIndex, bool kBf16, bool kHnd, int kThreads = 256>
+__global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
     const __half* __restrict__ q, const __half* __restrict__ kv_data,
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ sel_idx, int64_t sel_stride,
     uint32_t n_sel, __half* __restrict__ out, float* partial,
     uint32_t* __restrict__ counters, uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size,
     float scale_log2, uint32_t rows_per_split, uint32_t deferred_merge) {
-  __shared__ AttnShared sh;
+  constexpr int kGroups = kThreads / 16;  // rows in flight per load instruction of the workgroup
+  __shared__ AttnShared<kGroups> sh;
   const uint32_t split = blockIdx.x, n_split = gridDim.x;
   const uint32_t head = blockIdx.y;
   const uint32_t b = blockIdx.z;
@@ -551,6 +555,280 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_kernel(
   if (tid == 0) *counter = 0;  // ready for the next launch on this stream
 }
 
+
+// ---- dense decode attention with grouped queries on the matrix cores -------------------------------
+// The one GEMM-shaped piece of the path: a key/value head serves kG query heads, so the scores of a
+// tile of 16 tokens are a [16 tokens x 128] x [128 x kG] product and the weighted values a
+// [128 channels x 16 tokens] x [16 tokens x kG] product.  Both run as 16x16 MFMA tiles with the query
+// heads in the N dimension (kG of the 16 columns are used: the matrix cores have throughput to spare,
+// what matters is that the products leave the vector ALU, which the scalar kernel above keeps busy
+// with ~125 instructions per row and lane).
+//
+//   scores   S^T[token][head] = sum over four k-steps of v_mfma_f32_16x16x32: lane (t = lane % 16,
+//            qt = lane / 16) supplies the eight K channels 32j + 8qt .. +7 of token t for step j -
+//            exactly one 128-bit load of that token's row - and the same channels of query head
+//            lane % 16 (zero for the unused columns).  The order of the k index is the same on both
+//            sides, which is all the product needs.
+//   softmax  lane (head = lane % 16, qt) then holds the scores of tokens 4qt .. 4qt+3 of its head:
+//            fp32 online softmax, base 2; the running maximum is shared by the four lanes of a head,
+//            the denominator is kept per lane and summed at the end.
+//   values   O^T[channel][head] += V^T[channel][token] x P[token][head] as eight v_mfma_f32_16x16x16
+//            tiles.  P in the lane layout the score product left it in IS the B operand (tokens
+//            4qt .. 4qt+3 of head lane % 16).  The A operand wants four TOKENS of one channel per lane,
+//            memory has eight channels of one token per lane: the V tile goes through LDS (rows of
+//            264 bytes, so that the four token groups of a read fall into different banks).
+//
+// Workgroup = 8 waves = 8 query heads = 8 / kG key/value heads x kG token slices (wave w: key/value
+// head w % (8 / kG), slice w / (8 / kG)), so the merge of the slices and of the splits is the one of
+// the kernels above.  A wave walks over its tiles with the loads of the next tile and the page id of
+// the one after in flight.  grid = (splits, query heads / 8, batch).
+typedef _Float16 mfma_half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 mfma_half4 __attribute__((ext_vector_type(4)));
+typedef __bf16 mfma_bf8 __attribute__((ext_vector_type(8)));
+typedef short mfma_short4 __attribute__((ext_vector_type(4)));
+typedef float mfma_float4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kVtRowBytes = 264;                 // one token's 128 channels + 8 bytes
+constexpr uint32_t kVtWaveBytes = 16 * kVtRowBytes;   // a tile of 16 tokens
+
+template <bool kBf16>
+__device__ __forceinline__ mfma_float4 mfma_qk(const uint4& a, const uint4& b, mfma_float4 c) {
+  if (kBf16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const mfma_bf8*>(&a),
+                                                   *reinterpret_cast<const mfma_bf8*>(&b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const mfma_half8*>(&a),
+                                                *reinterpret_cast<const mfma_half8*>(&b), c, 0, 0, 0);
+}
+
+// a, b: four 16-bit values each, packed in two words
+template <bool kBf16>
+__device__ __forceinline__ mfma_float4 mfma_pv(const uint2& a, const uint2& b, mfma_float4 c) {
+  if (kBf16)
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const mfma_short4*>(&a),
+                                                     *reinterpret_cast<const mfma_short4*>(&b), c, 0,
+                                                     0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x16f16(*reinterpret_cast<const mfma_half4*>(&a),
+                                               *reinterpret_cast<const mfma_half4*>(&b), c, 0, 0, 0);
+}
+
+template <int kG>
+struct DenseGqaMfmaShared {
+  // the V tiles of the eight waves while they walk, the slice states once they are done
+  union {
+    alignas(16) unsigned char vt[8][kVtWaveBytes];
+    alignas(16) float o[kG][kDenseHeads][kHeadDim];
+  };
+  float m[kG][kDenseHeads];
+  float l[kG][kDenseHeads];
+  uint32_t is_last;
+};
+
+template <int kG, bool kBf16>
+__global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_mfma_kernel(
+    const __half* __restrict__ q, const __half* __restrict__ kv_data,
+    const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
+    const int32_t* __restrict__ seq_lens, __half* __restrict__ out, float* partial,
+    uint32_t* __restrict__ counters, uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size,
+    float scale_log2, uint32_t rows_per_split, KvLayout kvl) {
+  static_assert(kG == 2 || kG == 4 || kG == 8, "2, 4 or 8 query heads per key/value head");
+  constexpr int kKv = kDenseHeads / kG;   // key/value heads per workgroup
+  constexpr uint32_t kStep = 16u * kG;    // tokens between two tiles of a wave
+  __shared__ DenseGqaMfmaShared<kG> sh;
+  const uint32_t split = blockIdx.x, n_split = gridDim.x;
+  const uint32_t b = blockIdx.z;
+  const uint32_t tid = threadIdx.x;
+  const int lane = lane_id();
+  const int wave = wave_id_uniform();
+  const uint32_t kl = static_cast<uint32_t>(wave) % kKv;     // key/value head inside the workgroup
+  const uint32_t slice = static_cast<uint32_t>(wave) / kKv;  // token slice
+  const uint32_t t16 = static_cast<uint32_t>(lane) & 15u;    // token of the tile (loads), head (scores)
+  const uint32_t qt = static_cast<uint32_t>(lane) >> 4;      // channel quarter (loads), token group (scores)
+  const uint32_t kv_head = blockIdx.y * kKv + kl;
+  const uint32_t head0 = blockIdx.y * kDenseHeads;           // first query head of the workgroup
+
+  const int32_t seq_len = seq_lens[b];
+  const uint32_t row_begin = split * rows_per_split;
+  const uint32_t row_end = min(static_cast<uint32_t>(seq_len), row_begin + rows_per_split);
+  const int32_t* table = page_indices + page_indptr[b];
+  const uint32_t lp_last = seq_len > 0 ? (static_cast<uint32_t>(seq_len) - 1u) / page_size : 0u;
+  const __half* kv_lane = kv_data + static_cast<size_t>(kv_head) * kvl.head_stride + 8u * qt;
+
+  // B operand of the score product: channels 32j + 8qt .. +7 of query head t16 (columns >= kG: zero)
+  uint4 qb[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    qb[j] = make_uint4(0u, 0u, 0u, 0u);
+    if (t16 < kG)
+      qb[j] = *reinterpret_cast<const uint4*>(
+          q + (static_cast<size_t>(b) * num_heads + head0 + kl * kG + t16) * kHeadDim + 32 * j + 8 * qt);
+  }
+
+  mfma_float4 acc[8];  // acc[ct][i] = O[head t16][channel 16ct + 4qt + i]
+#pragma unroll
+  for (int ct = 0; ct < 8; ++ct) acc[ct] = mfma_float4{0.f, 0.f, 0.f, 0.f};
+  float m_run = kNegBig, l_run = 0.f;
+
+  unsigned char* vt = sh.vt[wave];
+  // page of the tile that starts at token `base` for this lane's token (clamped to the sequence)
+  auto page_of = [&](uint32_t base) __attribute__((always_inline)) -> uint32_t {
+    const uint32_t lp = min((base + t16) / page_size, lp_last);
+    return static_cast<uint32_t>(table[lp]);
+  };
+  // the eight loads of a tile: K and V channels 32j + 8qt .. +7 of token base + t16
+  auto issue = [&](uint32_t base, uint32_t page, uint4 (&kr)[4], uint4 (&vr)[4])
+                   __attribute__((always_inline)) {
+    const uint32_t r = min(base + t16, static_cast<uint32_t>(max(seq_len, 1)) - 1u);
+    const uint32_t lp = r / page_size;
+    const size_t row = static_cast<size_t>(page) * kvl.rows_per_page + (r - lp * page_size);
+    const __half* kp = kv_lane + row * kvl.tok_stride;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      kr[j] = *reinterpret_cast<const uint4*>(kp + 32 * j);
+      vr[j] = *reinterpret_cast<const uint4*>(kp + kvl.v_delta + 32 * j);
+    }
+  };
+  auto compute = [&](uint32_t base, const uint4 (&kr)[4], const uint4 (&vr)[4])
+                     __attribute__((always_inline)) {
+    mfma_float4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sc = mfma_qk<kBf16>(kr[j], qb[j], sc);
+    // the V tile on its way to the layout the second product wants (64-bit stores: rows are 8-byte
+    // aligned); the wave's LDS operations are carried out in order, no barrier needed
+    {
+      unsigned char* dst = vt + t16 * kVtRowBytes + 16u * qt;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        *reinterpret_cast<uint2*>(dst + 64 * j) = make_uint2(vr[j].x, vr[j].y);
+        *reinterpret_cast<uint2*>(dst + 64 * j + 8) = make_uint2(vr[j].z, vr[j].w);
+      }
+    }
+    float s[4];
+    bool ok[4];
+    float tmax = kNegBig;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ok[i] = base + 4u * qt + i < row_end;
+      s[i] = ok[i] ? sc[i] * scale_log2 : kNegBig;
+      tmax = fmaxf(tmax, s[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+    const float m_new = fmaxf(m_run, tmax);
+    const float alpha = exp2f(m_run - m_new);
+    float p[4], psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = ok[i] ? exp2f(s[i] - m_new) : 0.f;
+      psum += p[i];
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) {
+      acc[ct][0] *= alpha;
+      acc[ct][1] *= alpha;
+      acc[ct][2] *= alpha;
+      acc[ct][3] *= alpha;
+    }
+    const uint2 pb = make_uint2(pack2<kBf16>(p[0], p[1]), pack2<kBf16>(p[2], p[3]));
+    // A operand of tile ct: channel 16ct + t16 of tokens 4qt .. 4qt+3
+    const unsigned char* src = vt + 4u * qt * kVtRowBytes + 2u * t16;
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) {
+      uint32_t e[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        e[i] = *reinterpret_cast<const uint16_t*>(src + i * kVtRowBytes + 32 * ct);
+      const uint2 va = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
+      acc[ct] = mfma_pv<kBf16>(va, pb, acc[ct]);
+    }
+  };
+
+  // ---- the walk: compute tile i with the loads of tile i+1 and the page id of tile i+2 in flight ----
+  const uint32_t first = row_begin + slice * 16u;
+  if (first < row_end) {
+    uint4 k0[4], v0[4], k1[4], v1[4];
+    uint32_t page_next = page_of(first + kStep);
+    issue(first, page_of(first), k0, v0);
+    uint32_t base = first;
+    while (true) {
+      // even tile: registers 0
+      uint32_t page_after = page_of(base + 2 * kStep);
+      const bool more = base + kStep < row_end;
+      if (more) issue(base + kStep, page_next, k1, v1);
+      compute(base, k0, v0);
+      if (!more) break;
+      base += kStep;
+      page_next = page_after;
+      // odd tile: registers 1
+      page_after = page_of(base + 2 * kStep);
+      const bool more2 = base + kStep < row_end;
+      if (more2) issue(base + kStep, page_next, k0, v0);
+      compute(base, k1, v1);
+      if (!more2) break;
+      base += kStep;
+      page_next = page_after;
+    }
+  }
+
+  // ---- the slices of the workgroup, then the splits: as in dense_decode_gqa_kernel ------------------
+  __syncthreads();  // every wave is done with its V tile: the same LDS now takes the slice states
+  float l_tot = l_run;  // the four lanes of a head hold the denominators of their own tokens
+  l_tot += __shfl_xor(l_tot, 16);
+  l_tot += __shfl_xor(l_tot, 32);
+  if (t16 < kG) {
+    const uint32_t hl = kl * kG + t16;  // query head inside the workgroup
+    if (qt == 0) {
+      sh.m[slice][hl] = m_run;
+      sh.l[slice][hl] = l_tot;
+    }
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct)
+      *reinterpret_cast<float4*>(&sh.o[slice][hl][16 * ct + 4 * qt]) =
+          make_float4(acc[ct][0], acc[ct][1], acc[ct][2], acc[ct][3]);
+  }
+  __syncthreads();
+
+  const uint32_t hh = tid >> 6, cp = tid & 63u;  // thread -> (query head hh, channels 2cp and 2cp+1)
+  float M = kNegBig;
+#pragma unroll
+  for (int s2 = 0; s2 < kG; ++s2) M = fmaxf(M, sh.m[s2][hh]);
+  float L = 0.f, O0 = 0.f, O1 = 0.f;
+#pragma unroll
+  for (int s2 = 0; s2 < kG; ++s2) {
+    const float wgt = exp2f(sh.m[s2][hh] - M);
+    L += sh.l[s2][hh] * wgt;
+    O0 += sh.o[s2][hh][2 * cp] * wgt;
+    O1 += sh.o[s2][hh][2 * cp + 1] * wgt;
+  }
+  const size_t bh = static_cast<size_t>(b) * num_heads + head0 + hh;
+  uint32_t* orow = reinterpret_cast<uint32_t*>(out + bh * kHeadDim) + cp;
+  if (n_split == 1) {
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    *orow = pack2<kBf16>(O0 * inv, O1 * inv);
+    return;
+  }
+  float* mine = partial + (bh * kMaxSplits + split) * kPartialFloats;
+  if (cp == 0) store_partial_pair(mine, M, L);
+  store_partial_pair(mine + 2 + 2 * cp, O0, O1);
+  wait_own_stores();
+  __syncthreads();
+  uint32_t* counter = counters + static_cast<size_t>(b) * num_heads + head0;
+  if (tid == 0) {
+    const uint32_t prev = atomicAdd(counter, 1u);
+    sh.is_last = (prev == n_split - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!sh.is_last) return;
+  {
+    float LL, A[2];
+    merge_partial_pairs<32>(partial + bh * kMaxSplits * kPartialFloats, n_split, 2 * cp, LL, A);
+    const float inv = LL > 0.f ? 1.f / LL : 0.f;
+    *orow = pack2<kBf16>(A[0] * inv, A[1] * inv);
+  }
+  if (tid == 0) *counter = 0;  // ready for the next launch on this stream
+}
+
 }  // namespace adamas
 
 using namespace adamas;
@@ -568,7 +846,7 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
                               uint32_t num_heads, uint32_t num_kv_heads, uint32_t head_dim,
                               uint32_t page_size, float sm_scale, uint32_t max_seq_len,
                               adamas_stream_t stream, bool sel_is_rows, uint32_t flags) {
-  if (flags & ~(ADAMAS_F_BF16 | ADAMAS_F_HND)) return ADAMAS_E_BADARG;
+  if (flags & ~(ADAMAS_F_BF16 | ADAMAS_F_HND | ADAMAS_F_NO_MFMA)) return ADAMAS_E_BADARG;
   const bool bf16 = (flags & ADAMAS_F_BF16) != 0;
   const KvLayout lay = make_kv_layout((flags & ADAMAS_F_HND) != 0, page_size, num_kv_heads);
   if (sel_is_rows && !sel_idx) return ADAMAS_E_BADARG;
@@ -598,7 +876,11 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
     n_split = n_split > kMaxSplits ? kMaxSplits : n_split;
     uint32_t rows_per_split = (max_seq_len + n_split - 1) / n_split;
     rows_per_split = rows_per_split < 128 ? 128 : rows_per_split;
-    rows_per_split = (rows_per_split + kDenseRowsPerIter - 1) / kDenseRowsPerIter * kDenseRowsPerIter;
+    // whole tiles: 32 tokens per round of the vector kernels, 16 * group tokens (at most 128) per
+    // round of a workgroup of the matrix-core kernel
+    const bool gqa_mfma = gqa_kernel && !(flags & ADAMAS_F_NO_MFMA);
+    const uint32_t round_rows = gqa_mfma ? 128u : kDenseRowsPerIter;
+    rows_per_split = (rows_per_split + round_rows - 1) / round_rows * round_rows;
     n_split = (max_seq_len + rows_per_split - 1) / rows_per_split;
     float* partial = nullptr;
     uint32_t* counters = nullptr;
@@ -608,6 +890,28 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
       if (reinterpret_cast<uintptr_t>(workspace) & 255) return ADAMAS_E_ALIGN;
       counters = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + w.counters_off);
       partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + w.partial_off);
+    }
+    if (gqa_mfma) {
+#define ADAMAS_LAUNCH_DENSE_GQA_MFMA(G, BF)                                                      \
+  hipLaunchKernelGGL((dense_decode_gqa_mfma_kernel<G, BF>),                                      \
+                     dim3(n_split, num_heads / kDenseHeads, batch), dim3(kDenseThreads), 0,      \
+                     static_cast<hipStream_t>(stream), static_cast<const __half*>(q),            \
+                     static_cast<const __half*>(kv_data), page_indices, page_indptr, seq_lens,   \
+                     static_cast<__half*>(out), partial, counters, num_heads, num_kv_heads,      \
+                     page_size, scale_log2, rows_per_split, lay)
+      if (gq == 2) {
+        if (bf16) ADAMAS_LAUNCH_DENSE_GQA_MFMA(2, true);
+        else ADAMAS_LAUNCH_DENSE_GQA_MFMA(2, false);
+      } else if (gq == 4) {
+        if (bf16) ADAMAS_LAUNCH_DENSE_GQA_MFMA(4, true);
+        else ADAMAS_LAUNCH_DENSE_GQA_MFMA(4, false);
+      } else {
+        if (bf16) ADAMAS_LAUNCH_DENSE_GQA_MFMA(8, true);
+        else ADAMAS_LAUNCH_DENSE_GQA_MFMA(8, false);
+      }
+#undef ADAMAS_LAUNCH_DENSE_GQA_MFMA
+      ADAMAS_RETURN_IF_LAUNCH_FAILED();
+      return 0;
     }
     if (gqa_kernel) {
 #define ADAMAS_LAUNCH_DENSE_GQA(G, TILE, BF)                                                     \
@@ -645,12 +949,15 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
     return 0;
   }
   const uint32_t n_rows = sel_idx ? n_sel + 1u : max_seq_len;
-  // split so that the grid has a few thousand groups of work at most and every split has >= 128 rows
-  uint32_t rows_per_split = kRowsPerIter;
+  // one tile of rows per split (128, or 256 with the wide workgroup), more where that would take
+  // more than kMaxSplits splits
+  const bool wide = n_rows >= kWideRowsFrom;
+  const uint32_t rows_per_iter = (wide ? 32u : 16u) * kTile;
+  uint32_t rows_per_split = rows_per_iter;
   uint32_t n_split = (n_rows + rows_per_split - 1) / rows_per_split;
   if (n_split > kMaxSplits) {
-    rows_per_split = ((n_rows + kMaxSplits - 1) / kMaxSplits + kRowsPerIter - 1) / kRowsPerIter *
-                     kRowsPerIter;
+    rows_per_split = ((n_rows + kMaxSplits - 1) / kMaxSplits + rows_per_iter - 1) / rows_per_iter *
+                     rows_per_iter;
     n_split = (n_rows + rows_per_split - 1) / rows_per_split;
   }
   float* partial = nullptr;
@@ -664,18 +971,24 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
   }
   // from kDeferredMergeSplits splits on, the merge is a second short launch
   const uint32_t deferred = n_split >= kDeferredMergeSplits ? 1u : 0u;
-#define ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, HND)                                                    \
-  hipLaunchKernelGGL((sparse_decode_kernel<ROWS, BF, HND>), dim3(n_split, num_heads, batch),     \
-                     dim3(kAttnThreads), 0, static_cast<hipStream_t>(stream),                    \
+#define ADAMAS_LAUNCH_SPARSE_T(ROWS, BF, HND, T)                                                 \
+  hipLaunchKernelGGL((sparse_decode_kernel<ROWS, BF, HND, T>), dim3(n_split, num_heads, batch),  \
+                     dim3(T), 0, static_cast<hipStream_t>(stream),                               \
                      static_cast<const __half*>(q), static_cast<const __half*>(kv_data),         \
                      page_indices, page_indptr, seq_lens, sel_idx, sel_stride, n_sel,            \
                      static_cast<__half*>(out), partial, counters, num_heads, num_kv_heads,      \
                      page_size, scale_log2, rows_per_split, deferred)
+#define ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, HND)       \
+  if (wide) {                                       \
+    ADAMAS_LAUNCH_SPARSE_T(ROWS, BF, HND, 512);     \
+  } else {                                          \
+    ADAMAS_LAUNCH_SPARSE_T(ROWS, BF, HND, 256);     \
+  }
 #define ADAMAS_LAUNCH_SPARSE(ROWS, BF)        \
   if (flags & ADAMAS_F_HND) {                 \
-    ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, true);   \
+    ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, true)    \
   } else {                                    \
-    ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, false);  \
+    ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, false)   \
   }
   if (sel_is_rows) {
     if (bf16) {
@@ -692,6 +1005,7 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
   }
 #undef ADAMAS_LAUNCH_SPARSE
 #undef ADAMAS_LAUNCH_SPARSE_L
+#undef ADAMAS_LAUNCH_SPARSE_T
   ADAMAS_RETURN_IF_LAUNCH_FAILED();
   if (deferred) {
     if (bf16)

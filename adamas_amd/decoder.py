@@ -58,6 +58,36 @@ class DecoderConfig:
         return DecoderConfig(intermediate=14336, vocab=128256, rope_theta=500000.0, num_kv_heads=8)
 
 
+# Profiler ranges around the stages of the attention module, with the names the reference gives its
+# NVTX ranges (adamas/models/Adamas.py:112-220: "RoPE", "hadamard_transform", "append_kvh",
+# "prefill_attn", "full_attn", "estimate", "topk", "approx_attn", "o_proj").  On ROCm torch's nvtx
+# calls are roctx calls, so `rocprofv3 --marker-trace` shows them.  Where one launch covers several
+# of the reference's stages the range carries their names joined by "+".  Off by default: a range
+# is two host calls per stage and the eager decode loop is host-bound.
+_STAGE_RANGES = False
+
+
+def set_stage_ranges(enabled: bool) -> None:
+    global _STAGE_RANGES
+    _STAGE_RANGES = bool(enabled)
+
+
+class stage:
+    """`with stage("estimate+topk+approx_attn"):` = range_push / range_pop when ranges are on."""
+
+    def __init__(self, name: str):
+        self.name = name
+
+    def __enter__(self):
+        if _STAGE_RANGES:
+            torch.cuda.nvtx.range_push(self.name)
+
+    def __exit__(self, *exc):
+        if _STAGE_RANGES:
+            torch.cuda.nvtx.range_pop()
+        return False
+
+
 def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """x [N, K] @ w[M, K]^T.  One row goes through this package's matrix-vector kernel, which streams
     the weights faster than the library routines do for these shapes (measured for the 4096 x 11008
@@ -76,16 +106,20 @@ class AdamasAttention:
     def prefill(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, layer: int) -> torch.Tensor:
         """q, k, v [N, H, D] of a fresh sequence whose N positions are already reserved.  Appends K, V
         and codes (Hadamard inside the kernel), returns causal attention [N, H, D]."""
-        U.append_kvh(k, v, None, self.ctrl, layer)
-        o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None],
-                                           v.transpose(0, 1)[None], is_causal=True,
-                                           enable_gqa=k.shape[1] != q.shape[1])
-        return o[0].transpose(0, 1).contiguous()
+        with stage("hadamard_transform+append_kvh"):
+            U.append_kvh(k, v, None, self.ctrl, layer)
+        with stage("prefill_attn"):
+            o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None],
+                                               v.transpose(0, 1)[None], is_causal=True,
+                                               enable_gqa=k.shape[1] != q.shape[1])
+            return o[0].transpose(0, 1).contiguous()
 
     def decode(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, layer: int,
                sparse: bool) -> torch.Tensor:
         """q, k, v [B, H, D], one new token per sequence (its slot is reserved and counted)."""
-        return self.attend(q, U.append_kvh(k, v, None, self.ctrl, layer, q=q), layer, sparse)
+        with stage("hadamard_transform+append_kvh"):
+            q_code = U.append_kvh(k, v, None, self.ctrl, layer, q=q)
+        return self.attend(q, q_code, layer, sparse)
 
     def decode_from_qkv(self, qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, layer: int,
                         sparse: bool) -> torch.Tensor:
@@ -94,15 +128,19 @@ class AdamasAttention:
         c = self.ctrl
         if sparse and c.need_estimate() and U.layer_step_supported(c):
             # the append rides in the two launches of the step
-            return U.decode_layer_step(qkv, cos, sin, c, layer)
-        q, q_code = U.rope_append_decode(qkv, cos, sin, c, layer)
+            with stage("RoPE+hadamard_transform+append_kvh+estimate+topk+approx_attn"):
+                return U.decode_layer_step(qkv, cos, sin, c, layer)
+        with stage("RoPE+hadamard_transform+append_kvh"):
+            q, q_code = U.rope_append_decode(qkv, cos, sin, c, layer)
         return self.attend(q, q_code, layer, sparse)
 
     def attend(self, q: torch.Tensor, q_code: torch.Tensor, layer: int, sparse: bool) -> torch.Tensor:
         c = self.ctrl
         if sparse and c.need_estimate():
-            return U.decode_step(q, q_code, c, layer)
-        return U.decode_sparse_attn(q, c, layer, ALL_PAST_TOKENS)
+            with stage("estimate+topk+approx_attn"):
+                return U.decode_step(q, q_code, c, layer)
+        with stage("full_attn"):
+            return U.decode_sparse_attn(q, c, layer, ALL_PAST_TOKENS)
 
 
 class LlamaShapedDecoder:
@@ -183,8 +221,11 @@ class LlamaShapedDecoder:
         x = self.embed[token_ids]
         n = U.rms_norm_forward(x, self.layers[0]["attn_norm"], eps)
         for li, lw in enumerate(self.layers):
-            q, k, v = self._qkv(lw, n, start_pos=0)
-            d = F.linear(self.attn.prefill(q, k, v, li).view(n_tok, -1), lw["wo"])
+            with stage("RoPE"):
+                q, k, v = self._qkv(lw, n, start_pos=0)
+            o = self.attn.prefill(q, k, v, li)
+            with stage("o_proj"):
+                d = F.linear(o.view(n_tok, -1), lw["wo"])
             for s0 in range(0, n_tok, mlp_chunk):
                 xs = x[s0:s0 + mlp_chunk]
                 m = U.add_rms_norm(xs, d[s0:s0 + mlp_chunk], lw["mlp_norm"], eps)
@@ -205,7 +246,9 @@ class LlamaShapedDecoder:
             qkv = linear(n, lw["wqkv"]).view(-1, c.num_heads + 2 * c.kv_heads, c.head_dim)
             o = self.attn.decode_from_qkv(qkv, self.rope_cos, self.rope_sin, li,
                                           sparse and li >= c.dense_layers)
-            m = U.add_rms_norm(x, linear(o.view(1, -1), lw["wo"]), lw["mlp_norm"], eps)
+            with stage("o_proj"):
+                d = linear(o.view(1, -1), lw["wo"])
+            m = U.add_rms_norm(x, d, lw["mlp_norm"], eps)
             n = U.add_rms_norm(x, self._mlp(lw, m), self._next_norm(li), eps)
         return linear(n, self.lm_head)
 
@@ -239,7 +282,8 @@ class LlamaShapedDecoder:
             qkv = U.gemv_normed(wqkv_n, x, ps, eps).view(-1, c.num_heads + 2 * c.kv_heads, c.head_dim)
             o = self.attn.decode_from_qkv(qkv, self.rope_cos, self.rope_sin, li,
                                           sparse and li >= c.dense_layers)
-            U.gemv_add(lw["wo"], o.view(1, -1), x, ps)
+            with stage("o_proj"):
+                U.gemv_add(lw["wo"], o.view(1, -1), x, ps)
             U.gemv_add(lw["w_down"], U.gemv_normed(w_gate_up_n, x, ps, eps, gated=True), x, ps)
         return U.gemv_normed(fw["lm_head"], x, ps, eps)
 

@@ -108,6 +108,9 @@ def parse_args():
     ap.add_argument("--kv-heads", type=int, default=32,
                     help="key/value heads (grouped-query attention when below the 32 query heads); "
                          "the CPU baseline is skipped then")
+    ap.add_argument("--gqa-vector-alu", action="store_true",
+                    help="with --kv-heads below 32: time dense attention with the vector-ALU kernel "
+                         "(ADAMAS_F_NO_MFMA) instead of the matrix-core kernel")
     ap.add_argument("--kv-dtype", choices=("fp16", "bf16"), default="fp16",
                     help="16-bit format of q, K, V and the output (single-sequence workloads; the "
                          "reference and the headline figure are fp16)")
@@ -456,7 +459,7 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         ly = i % n_layers
         rc = lib.adamas_sparse_decode_f(q3.data_ptr(), kv_ptr[ly], tbl, indptr, lens, None, 0, 0,
                                         out.data_ptr(), ws.data_ptr(), ws.numel(), 1, H, Hkv, D, P,
-                                        sm_scale, L, kv_flags, _lib.current_stream())
+                                        sm_scale, L, dense_flags, _lib.current_stream())
         if rc:
             _lib.check(rc, "adamas_sparse_decode (dense)")
 
@@ -477,6 +480,7 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         if rc:
             _lib.check(rc, "adamas_step_attend")
 
+    dense_flags = kv_flags | (_lib.F_NO_MFMA if args.gqa_vector_alu else 0)
     k_new, v_new = k_dev[L - 1:].contiguous(), v_dev[L - 1:].contiguous()
     qc_tmp = torch.empty((1, H, 16), dtype=torch.int16, device=dev)
 

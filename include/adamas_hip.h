@@ -58,6 +58,9 @@ typedef void* adamas_stream_t;
 #define ADAMAS_F_BF16 2u           /* q, k, v, h and the KV cache hold bfloat16 instead of fp16          */
 #define ADAMAS_F_HND 4u            /* KV pages are [2][heads][page_size][128] instead of
                                       [2][page_size][heads][128]; the code cache keeps its layout      */
+#define ADAMAS_F_NO_MFMA 8u        /* adamas_sparse_decode_f, dense mode with 2, 4 or 8 query heads per
+                                      key/value head: the vector-ALU kernel instead of the matrix-core
+                                      one (same results within tolerance; kept for measurement)       */
 
 /* output formats of adamas_estimate / key modes of adamas_topk */
 #define ADAMAS_DIST_FP16 0u /* integer distance stored as fp16 (the reference's output dtype) */

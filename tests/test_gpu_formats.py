@@ -158,3 +158,46 @@ def test_step_bf16_ragged_batch(gpu_device, layout):
             assert ok, (i, h_bad)
             want = ora["out"]
         assert _close(o[i], want), i
+
+
+@pytest.mark.parametrize("dtype,layout", [(FP, NHD), (BF, NHD), (FP, HND)])
+@pytest.mark.parametrize("hq,hkv,page_size,kv_len", [
+    (32, 8, 16, 1), (32, 8, 16, 17), (32, 8, 16, 2049), (32, 8, 5, 1000), (32, 8, 16, 20000),
+    (32, 16, 16, 777), (32, 4, 16, 3001), (64, 8, 16, 513), (32, 4, 3, 130),
+])
+def test_dense_grouped_query_attention_on_matrix_cores(gpu_device, dtype, layout, hq, hkv, page_size,
+                                                       kv_len):
+    """Dense decode attention with 2, 4 or 8 query heads per key/value head: the matrix-core kernel
+    against the oracle on repeated heads, and against the vector-ALU kernel it replaced (flag
+    ADAMAS_F_NO_MFMA), on lengths that end inside a tile, inside a page and inside a split."""
+    import math
+    from adamas_amd import _lib
+    g = torch.Generator().manual_seed(kv_len * 7 + hq + hkv)
+    q = torch.randn(1, hq, 128, generator=g).to(dtype)
+    k = (torch.randn(kv_len, hkv, 128, generator=g) * 1.5).to(dtype)
+    v = torch.randn(kv_len, hkv, 128, generator=g).to(dtype)
+    cap = (kv_len + page_size - 1) // page_size * page_size
+    ctrl = T.make_controller(gpu_device, cap, 1 << 20, page_size, shuffle_seed=5, num_heads=hq,
+                             num_kv_heads=hkv, dtype=dtype, layout=layout)
+    T.fill_sequence(ctrl, k.to(gpu_device), v.to(gpu_device))
+    ctrl.inference_page_budget = 1 << 20
+    qd = q.to(gpu_device)
+    o = U.decode_sparse_attn(qd, ctrl, 0, U.ALL_PAST_TOKENS)
+    rep = hq // hkv
+    want = O.dense_attention(T.np16(q)[0], np.repeat(T.np16(k), rep, axis=1),
+                             np.repeat(T.np16(v), rep, axis=1))
+    assert _close(o[0], want)
+    assert torch.equal(o, U.decode_sparse_attn(qd, ctrl, 0, U.ALL_PAST_TOKENS))   # counters back at zero
+    # the vector-ALU kernel through the C ABI
+    lib = _lib.load()
+    o2 = torch.empty_like(qd)
+    ws = ctrl.workspace(1)
+    rc = lib.adamas_sparse_decode_f(
+        qd.data_ptr(), ctrl.pool.kv[0].data_ptr(), ctrl.seqs.table_dev.data_ptr(),
+        ctrl.seqs.indptr_dev.data_ptr(), ctrl.seqs.seq_lens_dev.data_ptr(), None, 0, 0, o2.data_ptr(),
+        ws.data_ptr(), ws.numel(), 1, hq, hkv, 128, page_size, 1.0 / math.sqrt(128), kv_len,
+        ctrl.kv_flags | _lib.F_NO_MFMA, _lib.current_stream())
+    assert rc == 0, _lib.error_string(rc)
+    assert _close(o2[0], want)
+    tol = 4e-3 if dtype == BF else 2e-3
+    assert (o.float() - o2.float()).abs().max().item() <= tol + 2.0 ** -7 * float(np.abs(want).max()) * (dtype == BF)
