@@ -227,42 +227,63 @@ __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
   if (tid == 0) counters[bh] = 0;  // ready for the next launch on this stream
 }
 
-// Merge of the split partials of sparse_decode_kernel as a launch of its own: grid (heads, batch), 128
-// threads = one per channel; plain loads, sixteen splits in flight per round.
+// Merge of the split partials as a launch of its own: grid (heads, batch), 512 threads = four groups
+// of one thread per channel; group g folds the splits g, g + 4, ... (plain loads, sixteen in flight
+// per round, so up to 64 splits cost one memory round trip), the four running states meet in LDS.
+constexpr int kMergeGroups = 4;
+
 template <bool kBf16>
-__global__ __launch_bounds__(kHeadDim) void merge_splits_kernel(const float* __restrict__ partial,
-                                                                __half* __restrict__ out,
-                                                                uint32_t num_heads,
-                                                                uint32_t n_split) {
+__global__ __launch_bounds__(kMergeGroups* kHeadDim) void merge_splits_kernel(
+    const float* __restrict__ partial, __half* __restrict__ out, uint32_t num_heads,
+    uint32_t n_split) {
+  __shared__ float sm[kMergeGroups][kHeadDim], sl[kMergeGroups][kHeadDim], sa[kMergeGroups][kHeadDim];
   const uint32_t bh = blockIdx.y * num_heads + blockIdx.x;
-  const uint32_t tid = threadIdx.x;
+  const uint32_t ch = threadIdx.x & (kHeadDim - 1);
+  const uint32_t grp = threadIdx.x / kHeadDim;
   const float* base = partial + static_cast<size_t>(bh) * kMaxSplits * kPartialFloats;
   float M = kNegBig, L = 0.f, A = 0.f;
-  for (uint32_t s0 = 0; s0 < n_split; s0 += 16) {
+  for (uint32_t s0 = grp; s0 < n_split; s0 += 16 * kMergeGroups) {
     float m[16], l[16], a[16];
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
-      const uint32_t s2 = min(s0 + u, n_split - 1);  // past the end: a duplicate, weighted zero below
+      // past the end: a duplicate of the last split, weighted zero below
+      const uint32_t s2 = min(s0 + u * kMergeGroups, n_split - 1);
       const float* p = base + static_cast<size_t>(s2) * kPartialFloats;
       m[u] = p[0];
       l[u] = p[1];
-      a[u] = p[2 + tid];
+      a[u] = p[2 + ch];
     }
     float m_new = M;
 #pragma unroll
-    for (int u = 0; u < 16; ++u) m_new = fmaxf(m_new, s0 + u < n_split ? m[u] : kNegBig);
+    for (int u = 0; u < 16; ++u)
+      m_new = fmaxf(m_new, s0 + u * kMergeGroups < n_split ? m[u] : kNegBig);
     const float keep = exp2f(M - m_new);
     L *= keep;
     A *= keep;
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
-      const float w = s0 + u < n_split ? exp2f(m[u] - m_new) : 0.f;
+      const float w = s0 + u * kMergeGroups < n_split ? exp2f(m[u] - m_new) : 0.f;
       L += l[u] * w;
       A += a[u] * w;
     }
     M = m_new;
   }
-  store_elem<kBf16>(out + static_cast<size_t>(bh) * kHeadDim + tid, L > 0.f ? A / L : 0.f);
+  sm[grp][ch] = M;
+  sl[grp][ch] = L;
+  sa[grp][ch] = A;
+  __syncthreads();
+  if (grp != 0) return;
+  float Mt = kNegBig;
+#pragma unroll
+  for (int g = 0; g < kMergeGroups; ++g) Mt = fmaxf(Mt, sm[g][ch]);
+  float Lt = 0.f, At = 0.f;
+#pragma unroll
+  for (int g = 0; g < kMergeGroups; ++g) {
+    const float w = exp2f(sm[g][ch] - Mt);  // a group without splits holds (kNegBig, 0, 0): weight 0 or 1 on zeros
+    Lt += sl[g][ch] * w;
+    At += sa[g][ch] * w;
+  }
+  store_elem<kBf16>(out + static_cast<size_t>(bh) * kHeadDim + ch, Lt > 0.f ? At / Lt : 0.f);
 }
 
 // ---- dense decode attention: every token of the sequence -----------------------------------------
@@ -277,10 +298,17 @@ constexpr int kDenseHeads = 8;
 constexpr int kDenseSlices = 4;
 constexpr int kDenseTile = 8;
 constexpr uint32_t kDenseRowsPerIter = kDenseSlices * kDenseTile;  // 32 tokens
-// Workgroups per launch.  Measured at 32K tokens x 32 heads: 128-160 workgroups (16-20 MB of loads
-// in flight) stream at 4.7 TB/s, 256 at 4.4, 512 at 3.5 and 64 at 3.1: beyond ~16 MB in flight the
-// memory system loses more to queueing than it gains in parallelism.
-constexpr uint32_t kDenseTargetBlocks = 128;
+// Workgroups per launch.  Measured at 32K tokens x 32 heads with the merge of the splits in a launch
+// of its own: 192 workgroups stream at 5.37 TB/s, 128 at 5.12, 256 at 5.31, 384 at 4.79, 512 at 5.12
+// (beyond ~24 MB in flight the memory system loses more to queueing than it gains in parallelism).
+// The grouped-query kernels read a fraction of the bytes per unit of work and want every CU busy.
+constexpr uint32_t kDenseTargetBlocks = 192;
+constexpr uint32_t kDenseGqaTargetBlocks = 256;
+// Splits from which the dense kernels leave the merge of their partials to a launch of its own.
+// Publishing partials inside the launch (write-through stores, their acknowledgement, the arrival
+// counter, the last workgroup's merge) sits at the end of every workgroup's critical path: with the
+// 64 splits of the grouped-query kernels it cost 10 us of 38, the extra launch costs 4.4.
+constexpr uint32_t kDenseDeferredSplits = 24;
 
 struct DenseShared {
   float m[kDenseSlices][kDenseHeads];
@@ -295,7 +323,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_kernel(
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ seq_lens, __half* __restrict__ out, float* partial,
     uint32_t* __restrict__ counters, uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size,
-    float scale_log2, uint32_t rows_per_split, KvLayout lay) {
+    float scale_log2, uint32_t rows_per_split, KvLayout lay, uint32_t deferred_merge) {
   __shared__ DenseShared sh;
   const uint32_t split = blockIdx.x, n_split = gridDim.x;
   const uint32_t hg = blockIdx.y;
@@ -360,6 +388,11 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_kernel(
   // several splits: publish the partial, the last workgroup of this head octet merges (same
   // agent-scope protocol as sparse_decode_kernel)
   float* mine = partial + (bh * kMaxSplits + split) * kPartialFloats;
+  if (deferred_merge) {  // many splits: plain stores, merged by merge_splits_kernel
+    if (cp == 0) *reinterpret_cast<float2*>(mine) = make_float2(M, L);
+    *reinterpret_cast<float2*>(mine + 2 + 2 * cp) = make_float2(O0, O1);
+    return;
+  }
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
   wait_own_stores();
@@ -422,7 +455,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_kernel(
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ seq_lens, __half* __restrict__ out, float* partial,
     uint32_t* __restrict__ counters, uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size,
-    float scale_log2, uint32_t rows_per_split, KvLayout kvl) {
+    float scale_log2, uint32_t rows_per_split, KvLayout kvl, uint32_t deferred_merge) {
   constexpr int kKv = DenseGqaShared<kG>::kKv;
   constexpr int kSlices = DenseGqaShared<kG>::kSlices;
   __shared__ DenseGqaShared<kG> sh;
@@ -535,6 +568,11 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_kernel(
     return;
   }
   float* mine = partial + (bh * kMaxSplits + split) * kPartialFloats;
+  if (deferred_merge) {  // many splits: plain stores, merged by merge_splits_kernel
+    if (cp == 0) *reinterpret_cast<float2*>(mine) = make_float2(M, L);
+    *reinterpret_cast<float2*>(mine + 2 + 2 * cp) = make_float2(O0, O1);
+    return;
+  }
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
   wait_own_stores();
@@ -629,7 +667,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_mfma_kernel(
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ seq_lens, __half* __restrict__ out, float* partial,
     uint32_t* __restrict__ counters, uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size,
-    float scale_log2, uint32_t rows_per_split, KvLayout kvl) {
+    float scale_log2, uint32_t rows_per_split, KvLayout kvl, uint32_t deferred_merge) {
   static_assert(kG == 2 || kG == 4 || kG == 8, "2, 4 or 8 query heads per key/value head");
   constexpr int kKv = kDenseHeads / kG;   // key/value heads per workgroup
   constexpr uint32_t kStep = 16u * kG;    // tokens between two tiles of a wave
@@ -744,30 +782,31 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_mfma_kernel(
     }
   };
 
-  // ---- the walk: compute tile i with the loads of tile i+1 and the page id of tile i+2 in flight ----
+  // ---- the walk: compute tile t with the loads of the next kAhead tiles and the page id of the one
+  // after them in flight (a ring of kAhead + 1 register buffers, indexed at compile time) ----------
+  constexpr int kAhead = 1;  // two tiles ahead measure the same, three slower (registers)
+  constexpr int kBuf = kAhead + 1;
   const uint32_t first = row_begin + slice * 16u;
   if (first < row_end) {
-    uint4 k0[4], v0[4], k1[4], v1[4];
-    uint32_t page_next = page_of(first + kStep);
-    issue(first, page_of(first), k0, v0);
-    uint32_t base = first;
-    while (true) {
-      // even tile: registers 0
-      uint32_t page_after = page_of(base + 2 * kStep);
-      const bool more = base + kStep < row_end;
-      if (more) issue(base + kStep, page_next, k1, v1);
-      compute(base, k0, v0);
-      if (!more) break;
-      base += kStep;
-      page_next = page_after;
-      // odd tile: registers 1
-      page_after = page_of(base + 2 * kStep);
-      const bool more2 = base + kStep < row_end;
-      if (more2) issue(base + kStep, page_next, k0, v0);
-      compute(base, k1, v1);
-      if (!more2) break;
-      base += kStep;
-      page_next = page_after;
+    const uint32_t n_tiles = (row_end - first + kStep - 1) / kStep;  // tiles of this wave
+    uint4 kr[kBuf][4], vr[kBuf][4];
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j)
+      if (static_cast<uint32_t>(j) < n_tiles)
+        issue(first + j * kStep, page_of(first + j * kStep), kr[j], vr[j]);
+    uint32_t page_next = page_of(first + kAhead * kStep);  // of the tile the first round issues
+    for (uint32_t t0 = 0; t0 < n_tiles; t0 += kBuf) {
+#pragma unroll
+      for (int sl = 0; sl < kBuf; ++sl) {
+        const uint32_t t = t0 + sl;
+        if (t >= n_tiles) break;
+        const uint32_t page_after = page_of(first + (t + kAhead + 1) * kStep);
+        if (t + kAhead < n_tiles)
+          issue(first + (t + kAhead) * kStep, page_next, kr[(sl + kAhead) % kBuf],
+                vr[(sl + kAhead) % kBuf]);
+        compute(first + t * kStep, kr[sl], vr[sl]);
+        page_next = page_after;
+      }
     }
   }
 
@@ -809,6 +848,15 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_mfma_kernel(
     return;
   }
   float* mine = partial + (bh * kMaxSplits + split) * kPartialFloats;
+  if (deferred_merge) {
+    // many splits: plain stores, the partials are merged by a launch of their own
+    // (merge_splits_kernel); publishing them inside the launch - write-through stores, their
+    // acknowledgement, the arrival counter, the last workgroup's merge - sat at the end of every
+    // workgroup's critical path and cost 10 us of 38 at 64 splits
+    if (cp == 0) *reinterpret_cast<float2*>(mine) = make_float2(M, L);
+    *reinterpret_cast<float2*>(mine + 2 + 2 * cp) = make_float2(O0, O1);
+    return;
+  }
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
   wait_own_stores();
@@ -871,7 +919,7 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
     const uint32_t groups = batch * (num_heads / kDenseHeads);
     // grouped queries read 1/gq of the bytes per unit of arithmetic: there the kernel is bound by
     // instruction issue, not by the memory system, and wants every CU busy
-    const uint32_t target_blocks = gqa_kernel ? 2 * kDenseTargetBlocks : kDenseTargetBlocks;
+    const uint32_t target_blocks = gqa_kernel ? kDenseGqaTargetBlocks : kDenseTargetBlocks;
     uint32_t n_split = (target_blocks + groups - 1) / groups;
     n_split = n_split > kMaxSplits ? kMaxSplits : n_split;
     uint32_t rows_per_split = (max_seq_len + n_split - 1) / n_split;
@@ -891,6 +939,21 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
       counters = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + w.counters_off);
       partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + w.partial_off);
     }
+    // from kDenseDeferredSplits splits on, the merge of the splits is a second short launch
+    const uint32_t deferred = n_split >= kDenseDeferredSplits ? 1u : 0u;
+    auto merge_launch = [&]() -> int {
+      if (!deferred) return 0;
+      if (bf16)
+        hipLaunchKernelGGL(merge_splits_kernel<true>, dim3(num_heads, batch),
+                           dim3(kMergeGroups * kHeadDim), 0, static_cast<hipStream_t>(stream),
+                           partial, static_cast<__half*>(out), num_heads, n_split);
+      else
+        hipLaunchKernelGGL(merge_splits_kernel<false>, dim3(num_heads, batch),
+                           dim3(kMergeGroups * kHeadDim), 0, static_cast<hipStream_t>(stream),
+                           partial, static_cast<__half*>(out), num_heads, n_split);
+      ADAMAS_RETURN_IF_LAUNCH_FAILED();
+      return 0;
+    };
     if (gqa_mfma) {
 #define ADAMAS_LAUNCH_DENSE_GQA_MFMA(G, BF)                                                      \
   hipLaunchKernelGGL((dense_decode_gqa_mfma_kernel<G, BF>),                                      \
@@ -898,7 +961,7 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
                      static_cast<hipStream_t>(stream), static_cast<const __half*>(q),            \
                      static_cast<const __half*>(kv_data), page_indices, page_indptr, seq_lens,   \
                      static_cast<__half*>(out), partial, counters, num_heads, num_kv_heads,      \
-                     page_size, scale_log2, rows_per_split, lay)
+                     page_size, scale_log2, rows_per_split, lay, deferred)
       if (gq == 2) {
         if (bf16) ADAMAS_LAUNCH_DENSE_GQA_MFMA(2, true);
         else ADAMAS_LAUNCH_DENSE_GQA_MFMA(2, false);
@@ -911,7 +974,7 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
       }
 #undef ADAMAS_LAUNCH_DENSE_GQA_MFMA
       ADAMAS_RETURN_IF_LAUNCH_FAILED();
-      return 0;
+      return merge_launch();
     }
     if (gqa_kernel) {
 #define ADAMAS_LAUNCH_DENSE_GQA(G, TILE, BF)                                                     \
@@ -920,7 +983,7 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
                      static_cast<hipStream_t>(stream), static_cast<const __half*>(q),            \
                      static_cast<const __half*>(kv_data), page_indices, page_indptr, seq_lens,   \
                      static_cast<__half*>(out), partial, counters, num_heads, num_kv_heads,      \
-                     page_size, scale_log2, rows_per_split, lay)
+                     page_size, scale_log2, rows_per_split, lay, deferred)
       if (gq == 2) {
         if (bf16) ADAMAS_LAUNCH_DENSE_GQA(2, 8, true);
         else ADAMAS_LAUNCH_DENSE_GQA(2, 8, false);
@@ -933,7 +996,7 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
       }
 #undef ADAMAS_LAUNCH_DENSE_GQA
       ADAMAS_RETURN_IF_LAUNCH_FAILED();
-      return 0;
+      return merge_launch();
     }
 #define ADAMAS_LAUNCH_DENSE(BF)                                                                  \
   hipLaunchKernelGGL(dense_decode_kernel<BF>, dim3(n_split, num_heads / kDenseHeads, batch),     \
@@ -941,12 +1004,12 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
                      static_cast<const __half*>(q), static_cast<const __half*>(kv_data),         \
                      page_indices, page_indptr, seq_lens, static_cast<__half*>(out), partial,    \
                      counters, num_heads, num_kv_heads, page_size, scale_log2, rows_per_split,   \
-                     lay)
+                     lay, deferred)
     if (bf16) ADAMAS_LAUNCH_DENSE(true);
     else ADAMAS_LAUNCH_DENSE(false);
 #undef ADAMAS_LAUNCH_DENSE
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
-    return 0;
+    return merge_launch();
   }
   const uint32_t n_rows = sel_idx ? n_sel + 1u : max_seq_len;
   // one tile of rows per split (128, or 256 with the wide workgroup), more where that would take
@@ -1009,11 +1072,11 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
   ADAMAS_RETURN_IF_LAUNCH_FAILED();
   if (deferred) {
     if (bf16)
-      hipLaunchKernelGGL(merge_splits_kernel<true>, dim3(num_heads, batch), dim3(kHeadDim), 0,
+      hipLaunchKernelGGL(merge_splits_kernel<true>, dim3(num_heads, batch), dim3(kMergeGroups * kHeadDim), 0,
                          static_cast<hipStream_t>(stream), partial, static_cast<__half*>(out),
                          num_heads, n_split);
     else
-      hipLaunchKernelGGL(merge_splits_kernel<false>, dim3(num_heads, batch), dim3(kHeadDim), 0,
+      hipLaunchKernelGGL(merge_splits_kernel<false>, dim3(num_heads, batch), dim3(kMergeGroups * kHeadDim), 0,
                          static_cast<hipStream_t>(stream), partial, static_cast<__half*>(out),
                          num_heads, n_split);
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
