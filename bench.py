@@ -493,6 +493,13 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         if rc:
             _lib.check(rc, "adamas_append_decode")
 
+    code_bytes_layer = ctrl.pool.codes[0].numel() * 2
+
+    def k_read(i):   # a launch that only reads one layer's code cache
+        rc = lib.adamas_read_probe(code_ptr[i % n_layers], code_bytes_layer, None, _lib.current_stream())
+        if rc:
+            _lib.check(rc, "adamas_read_probe")
+
     # ---- warm-up (untimed) ----
     for i in range(args.warmup):
         step(i)
@@ -507,14 +514,15 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         for i in range(args.steps):
             step(i)
         torch.cuda.synchronize()
-        for fn in (k_estimate, k_topk, k_attn, k_append):
+        for fn in (k_estimate, k_topk, k_attn, k_append, k_read):
             for i in range(16):
                 fn(i)
         for i in range(4):
             k_dense(i)
         torch.cuda.synchronize()
         print(json.dumps({"profile_run": True, "steps": args.steps, "workload": w.name,
-                          "calibration_copy_bytes": 256 << 20}), flush=True)
+                          "calibration_copy_bytes": 256 << 20,
+                          "kernel_sources_digest": kernel_sources_digest()}), flush=True)
         return None
 
     # ---- eager K steps (host launch overhead included), for the record ----
@@ -559,13 +567,6 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
     dense_us = time_graph(torch, k_dense, max(16, k_iters // 8), flush=flush)
     dense_gbps = 2 * L * Hkv * D * 2 / (dense_us * 1e-6) / 1e9
     # the practical ceiling: a kernel that only reads the same rotated code caches, in this run
-    code_bytes_layer = ctrl.pool.codes[0].numel() * 2
-
-    def k_read(i):
-        rc = lib.adamas_read_probe(code_ptr[i % n_layers], code_bytes_layer, None, _lib.current_stream())
-        if rc:
-            _lib.check(rc, "adamas_read_probe")
-
     read_us = time_graph(torch, k_read, k_iters, flush=flush)
     log(f"step kernels: estimate+select {cand_us:.2f} us (cache-hot {cand_hot_us:.2f}), "
         f"select+attend {attend_us:.2f}; plain read of one code cache {read_us:.2f} us "
