@@ -114,6 +114,9 @@ def parse_args():
     ap.add_argument("--kv-dtype", choices=("fp16", "bf16"), default="fp16",
                     help="16-bit format of q, K, V and the output (single-sequence workloads; the "
                          "reference and the headline figure are fp16)")
+    ap.add_argument("--kv-layout", choices=("nhd", "hnd"), default="nhd",
+                    help="page layout of the KV cache: [2, page, heads, 128] (the reference's) or "
+                         "[2, heads, page, 128]")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time box of the CPU baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-e2e", action="store_true",
@@ -386,9 +389,10 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
     order = np.random.default_rng(w.seed).permutation(n_pages).tolist()   # non-contiguous pages
     bf16 = args.kv_dtype == "bf16"
     fdt = torch.bfloat16 if bf16 else torch.float16
-    kv_flags = _lib.dtype_flags(fdt)   # the *_f entry points with flags 0 are the plain ones
+    layout = U.TensorLayout.HND if args.kv_layout == "hnd" else U.TensorLayout.NHD
     ctrl = U.InferenceController(n_layers, H, D, P, budget, L, fdt, dev, page_order=order,
-                                 num_kv_heads=Hkv)
+                                 num_kv_heads=Hkv, layout=layout)
+    kv_flags = ctrl.kv_flags   # the *_f entry points with flags 0 are the plain ones
     k_dev, v_dev, q_dev = (seq.k[:, :Hkv].to(dev).to(fdt), seq.v[:, :Hkv].to(dev).to(fdt),
                            seq.q.to(dev).to(fdt))
     chunk = 8192
@@ -652,7 +656,8 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         "data": "synthetic",
         "config": {"workload": w.name, "batch": 1, "heads": H, "kv_heads": Hkv, "head_dim": D,
                    "kv_len": L,
-                   "page_size": P, "token_budget": budget, "rotated_layer_caches": n_layers,
+                   "page_size": P, "kv_layout": args.kv_layout.upper(), "token_budget": budget,
+                   "rotated_layer_caches": n_layers,
                    "timed_region": "HIP graph of K steps",
                    "launches_per_step": 2 if fused else 3},
         "achieved_hbm_GBps": round(step_bytes / (step_us * 1e-6) / 1e9, 1),
