@@ -119,6 +119,30 @@ def test_sparse_selection_keeps_output_close_when_budget_is_generous(model, gpu_
     assert _close(res[1], res[0], tol=0.25)
 
 
+def test_stage_ranges_do_not_change_results(model, gpu_device):
+    """Profiler ranges around the stages (the reference's NVTX names) are host calls only: prefill
+    logits and the eager sparse decode give the same bits with them on, and the graph loop still
+    captures and replays."""
+    from adamas_amd import decoder as D
+    ids = _prompt(gpu_device)
+    res = []
+    for on in (False, True):
+        D.set_stage_ranges(on)
+        try:
+            model.init_cache(page_size=16, max_seq_len=512, token_budget=64)
+            logits = model.prefill(ids)
+            first = logits.argmax(-1)
+            step = model.decode_step_eager(first, sparse=True).clone()
+            toks, _ = model.generate(step.argmax(-1), 4, sparse=True, use_graph=True)
+            res.append((logits.clone(), step, toks.numpy().copy()))
+            model.clear()
+        finally:
+            D.set_stage_ranges(False)
+    assert torch.equal(res[0][0], res[1][0])
+    assert torch.equal(res[0][1], res[1][1])
+    assert np.array_equal(res[0][2], res[1][2])
+
+
 # ------------------------------------------------------- the one-launch operators of the decoder --
 @pytest.mark.parametrize("rows,hidden", [(1, 4096), (7, 4096), (300, 512), (3, 11008)])
 def test_rmsnorm_matches_torch(gpu_device, rows, hidden):
