@@ -12,6 +12,11 @@ namespace adamas {
 
 constexpr float kNegBig = -1.0e30f;
 
+// 2^x as the bare hardware instruction.  The library routine exp2f() wraps it in five more instructions that only matter
+// for results below 2^-126, which are weights of zero here; for every other argument the bits are
+// the same.  The attention kernels are bound by instruction issue, and a softmax has many of these.
+__device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+
 template <bool kBf16 = false>
 __device__ __forceinline__ void unpack8(uint4 r, float f[8]) {
   const uint32_t w[4] = {r.x, r.y, r.z, r.w};
@@ -45,7 +50,8 @@ struct HeadKV {
   const __half* kv_data;   // page pool of the layer
   const int32_t* table;    // page table of the sequence
   size_t head_off;         // offset of the head (see above) + 8 * lane_in_group
-  size_t tok_stride;       // elements between adjacent slots of a page
+  uint32_t tok_stride;     // elements between adjacent slots of a page (32 bits: row * tok_stride
+                           // is then one 32 x 32 -> 64 bit multiply-add per row address)
   size_t v_delta;          // K -> V inside a page
   uint32_t row_mult;       // rows per page
   uint32_t page_size;
@@ -80,7 +86,7 @@ __device__ __forceinline__ void set_kv_layout_static(HeadKV& kv, uint32_t kv_hea
     kv.row_mult = 2u * page_size * num_kv_heads;
     kv.v_delta = static_cast<size_t>(page_size) * num_kv_heads * kHeadDim;
   } else {
-    kv.tok_stride = static_cast<size_t>(num_kv_heads) * kHeadDim;
+    kv.tok_stride = num_kv_heads * kHeadDim;
     kv.head_off = static_cast<size_t>(kv_head) * kHeadDim + 8 * c;
     kv.row_mult = 2u * page_size;
     kv.v_delta = static_cast<size_t>(page_size) * kv.tok_stride;
@@ -110,30 +116,43 @@ struct SoftmaxState {
 //                       translated through the page table;
 //   kRowIndex == true : pos_of gives the K row index page*row_mult + slot directly (negative =
 //                       skip), no table access.
-template <int kGroups, int kTile, bool kRowIndex = false, bool kBf16 = false, typename PosFn>
+//   kAllValid (with kRowIndex): every list entry is a valid row index; slots past row_end then load
+//                       the last row of the list again (its weight is zero) instead of branching
+//                       around the loads.
+template <int kGroups, int kTile, bool kRowIndex = false, bool kBf16 = false, bool kAllValid = false,
+          typename PosFn>
 __device__ __forceinline__ void attend_rows(const HeadKV& kv, const float (&qf)[8], uint32_t g,
                                             uint32_t row_begin, uint32_t row_end, PosFn&& pos_of,
                                             SoftmaxState& st) {
+  static_assert(!kAllValid || kRowIndex, "kAllValid is for lists of row indices");
   for (uint32_t base = row_begin; base < row_end; base += kGroups * kTile) {
     uint4 kr[kTile], vr[kTile];
     bool valid[kTile];
 #pragma unroll
     for (int i = 0; i < kTile; ++i) {
       const uint32_t r = base + i * kGroups + g;
+      if (kAllValid) {
+        valid[i] = r < row_end;
+        const uint32_t row = static_cast<uint32_t>(pos_of(min(r, row_end - 1u)));
+        const __half* kp = kv.kv_data + static_cast<size_t>(row) * kv.tok_stride + kv.head_off;
+        kr[i] = *reinterpret_cast<const uint4*>(kp);
+        vr[i] = *reinterpret_cast<const uint4*>(kp + kv.v_delta);
+        continue;
+      }
       const int32_t pos = (r < row_end) ? pos_of(r) : -1;
       valid[i] = pos >= 0 && (kRowIndex || pos < kv.seq_len);
       kr[i] = make_uint4(0, 0, 0, 0);
       vr[i] = make_uint4(0, 0, 0, 0);
       if (valid[i]) {
-        size_t row;
+        uint32_t row;  // K row indices are below 2^31 everywhere (the row lists are int32)
         if (kRowIndex) {
-          row = static_cast<size_t>(pos);
+          row = static_cast<uint32_t>(pos);
         } else {
           const uint32_t lp = static_cast<uint32_t>(pos) / kv.page_size;
           const uint32_t slot = static_cast<uint32_t>(pos) - lp * kv.page_size;
-          row = static_cast<size_t>(kv.table[lp]) * kv.row_mult + slot;
+          row = static_cast<uint32_t>(kv.table[lp]) * kv.row_mult + slot;
         }
-        const __half* kp = kv.kv_data + row * kv.tok_stride + kv.head_off;
+        const __half* kp = kv.kv_data + static_cast<size_t>(row) * kv.tok_stride + kv.head_off;
         kr[i] = *reinterpret_cast<const uint4*>(kp);
         vr[i] = *reinterpret_cast<const uint4*>(kp + kv.v_delta);
       }
@@ -151,13 +170,13 @@ __device__ __forceinline__ void attend_rows(const HeadKV& kv, const float (&qf)[
       s[i] = valid[i] ? d : kNegBig;
       m_new = fmaxf(m_new, s[i]);
     }
-    const float alpha = exp2f(st.m - m_new);
+    const float alpha = exp2_raw(st.m - m_new);
     st.l *= alpha;
 #pragma unroll
     for (int j = 0; j < 8; ++j) st.o[j] *= alpha;
 #pragma unroll
     for (int i = 0; i < kTile; ++i) {
-      const float p = valid[i] ? exp2f(s[i] - m_new) : 0.f;
+      const float p = valid[i] ? exp2_raw(s[i] - m_new) : 0.f;
       st.l += p;
       float vf[8];
       unpack8<kBf16>(vr[i], vf);
@@ -183,7 +202,7 @@ __device__ __forceinline__ void fold_state(SoftmaxState& st, int delta) {
   const float m_o = __shfl_xor(st.m, delta);
   const float l_o = __shfl_xor(st.l, delta);
   const float m_n = fmaxf(st.m, m_o);
-  const float a = exp2f(st.m - m_n), b = exp2f(m_o - m_n);
+  const float a = exp2_raw(st.m - m_n), b = exp2_raw(m_o - m_n);
   st.l = st.l * a + l_o * b;
 #pragma unroll
   for (int j = 0; j < 8; ++j) st.o[j] = st.o[j] * a + __shfl_xor(st.o[j], delta) * b;
@@ -217,7 +236,7 @@ __device__ __forceinline__ void merge_groups(SoftmaxState st, uint32_t g, uint32
     for (int i = 0; i < kWavesM; ++i) M = fmaxf(M, sh.m[i]);
 #pragma unroll
     for (int i = 0; i < kWavesM; ++i) {
-      const float wgt = exp2f(sh.m[i] - M);
+      const float wgt = exp2_raw(sh.m[i] - M);
       L += sh.l[i] * wgt;
       O += sh.o[i][tid] * wgt;
     }

@@ -50,13 +50,13 @@ __device__ __forceinline__ void merge_partials(const float* base, uint32_t n_spl
     float m_new = M;
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) m_new = fmaxf(m_new, s0 + u < n_split ? m[u] : kNegBig);
-    const float keep = exp2f(M - m_new);
+    const float keep = exp2_raw(M - m_new);
     L *= keep;
 #pragma unroll
     for (int e = 0; e < kVec; ++e) A[e] *= keep;
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
-      const float w = s0 + u < n_split ? exp2f(m[u] - m_new) : 0.f;
+      const float w = s0 + u < n_split ? exp2_raw(m[u] - m_new) : 0.f;
       L += l[u] * w;
 #pragma unroll
       for (int e = 0; e < kVec; ++e) A[e] += a[u][e] * w;
@@ -93,14 +93,14 @@ __device__ __forceinline__ void merge_partial_pairs(const float* base, uint32_t 
 #pragma unroll
     for (int u = 0; u < kBatch; ++u)
       m_new = fmaxf(m_new, s0 + u < n_split ? __uint_as_float(static_cast<uint32_t>(ml[u])) : kNegBig);
-    const float keep = exp2f(M - m_new);
+    const float keep = exp2_raw(M - m_new);
     L *= keep;
     A[0] *= keep;
     A[1] *= keep;
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       const float w = s0 + u < n_split
-                          ? exp2f(__uint_as_float(static_cast<uint32_t>(ml[u])) - m_new)
+                          ? exp2_raw(__uint_as_float(static_cast<uint32_t>(ml[u])) - m_new)
                           : 0.f;
       L += __uint_as_float(static_cast<uint32_t>(ml[u] >> 32)) * w;
       A[0] += __uint_as_float(static_cast<uint32_t>(aa[u])) * w;
@@ -259,12 +259,12 @@ __global__ __launch_bounds__(kMergeGroups* kHeadDim) void merge_splits_kernel(
 #pragma unroll
     for (int u = 0; u < 16; ++u)
       m_new = fmaxf(m_new, s0 + u * kMergeGroups < n_split ? m[u] : kNegBig);
-    const float keep = exp2f(M - m_new);
+    const float keep = exp2_raw(M - m_new);
     L *= keep;
     A *= keep;
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
-      const float w = s0 + u * kMergeGroups < n_split ? exp2f(m[u] - m_new) : 0.f;
+      const float w = s0 + u * kMergeGroups < n_split ? exp2_raw(m[u] - m_new) : 0.f;
       L += l[u] * w;
       A += a[u] * w;
     }
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kMergeGroups* kHeadDim) void merge_splits_kernel(
   float Lt = 0.f, At = 0.f;
 #pragma unroll
   for (int g = 0; g < kMergeGroups; ++g) {
-    const float w = exp2f(sm[g][ch] - Mt);  // a group without splits holds (kNegBig, 0, 0): weight 0 or 1 on zeros
+    const float w = exp2_raw(sm[g][ch] - Mt);  // a group without splits holds (kNegBig, 0, 0): weight 0 or 1 on zeros
     Lt += sl[g][ch] * w;
     At += sa[g][ch] * w;
   }
@@ -374,7 +374,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_kernel(
   float L = 0.f, O0 = 0.f, O1 = 0.f;
 #pragma unroll
   for (int s2 = 0; s2 < kDenseSlices; ++s2) {
-    const float wgt = exp2f(sh.m[s2][hh] - M);
+    const float wgt = exp2_raw(sh.m[s2][hh] - M);
     L += sh.l[s2][hh] * wgt;
     O0 += sh.o[s2][hh][2 * cp] * wgt;
     O1 += sh.o[s2][hh][2 * cp + 1] * wgt;
@@ -519,13 +519,13 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_kernel(
         sc[i] = valid[i] ? d : kNegBig;
         m_new = fmaxf(m_new, sc[i]);
       }
-      const float alpha = exp2f(st[j].m - m_new);
+      const float alpha = exp2_raw(st[j].m - m_new);
       st[j].l *= alpha;
 #pragma unroll
       for (int e = 0; e < 8; ++e) st[j].o[e] *= alpha;
 #pragma unroll
       for (int i = 0; i < kTile; ++i) {
-        const float pw = valid[i] ? exp2f(sc[i] - m_new) : 0.f;
+        const float pw = valid[i] ? exp2_raw(sc[i] - m_new) : 0.f;
         st[j].l += pw;
         float vf[8];
         unpack8<kBf16>(vr[i], vf);
@@ -557,7 +557,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_kernel(
   float L = 0.f, O0 = 0.f, O1 = 0.f;
 #pragma unroll
   for (int s2 = 0; s2 < kSlices; ++s2) {
-    const float wgt = exp2f(sh.m[s2][hh] - M);
+    const float wgt = exp2_raw(sh.m[s2][hh] - M);
     L += sh.l[s2][hh] * wgt;
     O0 += sh.o[s2][hh][2 * cp] * wgt;
     O1 += sh.o[s2][hh][2 * cp + 1] * wgt;
@@ -754,11 +754,11 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_mfma_kernel(
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
     const float m_new = fmaxf(m_run, tmax);
-    const float alpha = exp2f(m_run - m_new);
+    const float alpha = exp2_raw(m_run - m_new);
     float p[4], psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      p[i] = ok[i] ? exp2f(s[i] - m_new) : 0.f;
+      p[i] = ok[i] ? exp2_raw(s[i] - m_new) : 0.f;
       psum += p[i];
     }
     l_run = l_run * alpha + psum;
@@ -837,7 +837,7 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_mfma_kernel(
   float L = 0.f, O0 = 0.f, O1 = 0.f;
 #pragma unroll
   for (int s2 = 0; s2 < kG; ++s2) {
-    const float wgt = exp2f(sh.m[s2][hh] - M);
+    const float wgt = exp2_raw(sh.m[s2][hh] - M);
     L += sh.l[s2][hh] * wgt;
     O0 += sh.o[s2][hh][2 * cp] * wgt;
     O1 += sh.o[s2][hh][2 * cp + 1] * wgt;

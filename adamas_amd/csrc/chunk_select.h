@@ -173,8 +173,10 @@ struct FinalSelectShared {
 
 // Level 2 for one row, called by all 512 threads of the workgroup.  crow: the row's n_slots =
 // n_chunks * cand_stride candidate slots (n_slots <= 512 * 8 * kGroups, cand_stride a multiple of 8);
-// hist_rows: its n_chunks histogram rows of 512 bytes.  emit(pos, chunk, offset, key, payload) is
-// called once per selected candidate, pos in [0, n_take), in the lane that holds it.  Returns n_take
+// hist_rows: its n_chunks histogram rows of 512 bytes.  emit(pos, slot0, offset, key, payload) is
+// called once per selected candidate, pos in [0, n_take), in the lane that holds it; slot0 is the
+// first slot of the candidate's group of 8 (its chunk is slot0 / cand_stride), offset its token
+// offset inside the chunk.  Returns n_take
 // (k, or the number of candidates if smaller).  Ends without a barrier: the caller synchronises
 // before it reads what emit() wrote.
 // while_loading() is called once by every thread after the loads of the histogram rows and of the
@@ -255,7 +257,9 @@ __device__ __forceinline__ uint32_t final_select(const uint64_t* __restrict__ cr
     }
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      keys[j * 8 + r] = c[r] == kEmptyCand64 ? kInvalidKey : static_cast<uint32_t>(c[r] >> 48);
+      // an unused slot is all ones: its key field reads 0xffff, above every threshold (<= 512), so it
+      // needs no test of its own
+      keys[j * 8 + r] = static_cast<uint32_t>(c[r] >> 48);
       krow[j * 8 + r] = static_cast<uint32_t>(c[r]);
     }
 #pragma unroll
@@ -332,12 +336,13 @@ __device__ __forceinline__ uint32_t final_select(const uint64_t* __restrict__ cr
 #pragma unroll
   for (int j = 0; j < kGroups; ++j) {
     const uint32_t bj[2] = {below[2 * j], below[2 * j + 1]}, ej[2] = {equal[2 * j], equal[2 * j + 1]};
-    // cand_stride is a multiple of 8: the 8 slots of a group belong to one chunk
-    const uint32_t chunk_of = block_item_index<kItems>(wave, lane, j, 0) / cand_stride;
+    // cand_stride is a multiple of 8: the 8 slots of a group belong to one chunk, slot0 / cand_stride
+    // (left to the caller: a division per lane that only a caller who wants positions has to pay)
+    const uint32_t slot0 = block_item_index<kItems>(wave, lane, j, 0);
     lane_emit<2>(bj, ej, n_below, quota, base_b + (ex[j] & 0xffffu), base_e + (ex[j] >> 16),
                  [&](uint32_t pos, int i) __attribute__((always_inline)) {
                    const uint32_t tk = toks[j * 4 + (i >> 1)];
-                   emit(pos, chunk_of, (i & 1) ? (tk >> 16) : (tk & 0xffffu), keys[j * 8 + i],
+                   emit(pos, slot0, (i & 1) ? (tk >> 16) : (tk & 0xffffu), keys[j * 8 + i],
                         krow[j * 8 + i]);
                  });
     base_b += tot[j] & 0xffffu;

@@ -320,7 +320,7 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
 struct SelectAttendShared {
   MergeShared<32> merge;
   int32_t rows[kFusedMaxSel + 1];     // K row index of every selected token, then the current one
-  int32_t sel_pos[kFusedMaxSel + 1];  // logical position of every selected token
+  int32_t sel_pos[kFusedMaxSel + 1];  // of every selected token: first slot of its group << 16 | offset in its chunk
   FinalSelectShared sel;
   // kFromQkv: the rotated query (scaled for the softmax), the rotated new key and the new value
   alignas(16) float qkv_now[3][kHeadDim];
@@ -420,10 +420,12 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   const uint32_t n_take = final_select<kGroups>(
       crow, n_slots, hist + static_cast<size_t>(bh) * hist_stride * kHistBins, n_chunks, k,
       cand_stride, sh.sel,
-      [&](uint32_t pos, uint32_t chunk_of, uint32_t offset, uint32_t, uint32_t krow)
+      [&](uint32_t pos, uint32_t slot0, uint32_t offset, uint32_t, uint32_t krow)
           __attribute__((always_inline)) {
             sh.rows[pos] = static_cast<int32_t>(krow);
-            sh.sel_pos[pos] = static_cast<int32_t>(chunk_of * chunk_tokens + offset);
+            // slot (< 2^15) and offset in the chunk (< 2^16): turned into a position only when
+            // the caller asked for the selection
+            sh.sel_pos[pos] = static_cast<int32_t>((slot0 << 16) | offset);
           },
       [&]() __attribute__((always_inline)) {
         if (kFromQkv) make_q_and_key();
@@ -433,7 +435,12 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   __syncthreads();
   // the selection goes out once the row list is complete (every wave has emitted its part)
   if (sdst)
-    for (uint32_t i = tid; i < k; i += kAttThreads) sdst[i] = i < n_take ? sh.sel_pos[i] : -1;
+    for (uint32_t i = tid; i < k; i += kAttThreads) {
+      const uint32_t v = static_cast<uint32_t>(sh.sel_pos[i]);
+      sdst[i] = i < n_take
+                    ? static_cast<int32_t>((v >> 16) / cand_stride * chunk_tokens + (v & 0xffffu))
+                    : -1;
+    }
   if (kFromQkv) {
     // the query for every group, the new key and value for the group that attends them
     const float4 a0 = *reinterpret_cast<const float4*>(&sh.qkv_now[0][8 * c16]);
@@ -471,7 +478,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   set_kv_layout_static<kHnd>(kv, head / (num_heads / num_kv_heads), c16, num_kv_heads, page_size);
   kv.seq_len = seq_len;
   SoftmaxState st;
-  attend_rows<32, 5, true, kBf16>(kv, qf, g, 0u, kFromQkv ? n_take : n_take + 1u,
+  attend_rows<32, 4, true, kBf16, true>(kv, qf, g, 0u, kFromQkv ? n_take : n_take + 1u,
                            [&](uint32_t r) __attribute__((always_inline)) -> int32_t {
                              return sh.rows[r];
                            },
@@ -484,8 +491,8 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     d = group16_sum(d);
     const bool mine = g == 0;
     const float m_new = mine ? fmaxf(st.m, d) : st.m;
-    const float alpha = exp2f(st.m - m_new);
-    const float pw = mine ? exp2f(d - m_new) : 0.f;
+    const float alpha = exp2_raw(st.m - m_new);
+    const float pw = mine ? exp2_raw(d - m_new) : 0.f;
     st.l = st.l * alpha + pw;
 #pragma unroll
     for (int j = 0; j < 8; ++j) st.o[j] = st.o[j] * alpha + pw * vcur[j];
