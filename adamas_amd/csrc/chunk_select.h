@@ -89,8 +89,9 @@ __device__ __forceinline__ void raw_class_masks(const uint32_t (&keys)[kItems], 
 // One wave: the k smallest of its 64 x kItems keys (lane l holds items kItems*l .. kItems*l + kItems-1,
 // kInvalidKey = no item; n_valid = number of items).  dst: the chunk's candidate list (cand_stride
 // slots, unused ones are filled with kEmptyCand64); hrow: this lane's 8 bytes of the chunk's
-// histogram row; hist_lds: 256 words of LDS owned by this wave, 16-byte aligned; payload(item) -> 32
-// bits stored with the candidate (evaluated for selected items only).
+// histogram row; hist_lds: 256 words of LDS owned by this wave, 16-byte aligned; payload(item, i) -> 32
+// bits stored with the candidate (evaluated for selected items only; i = item - kItems * lane is a
+// constant at every call, so a caller can keep its payloads in registers).
 // The threshold is read off a histogram instead of being searched for: every lane counts its keys
 // into 512 bins of 16-bit counters in LDS, a prefix sum over the bins (8 bins per lane, DPP scan
 // across the lanes) finds the bin that holds the k-th smallest key, and the histogram of the
@@ -159,7 +160,7 @@ __device__ __forceinline__ void chunk_select_emit(const uint32_t (&keys)[kItems]
                         [&](uint32_t pos, int i) __attribute__((always_inline)) {
                           const uint32_t tok = static_cast<uint32_t>(lane) * kItems + i;
                           dst[pos] =
-                              (static_cast<uint64_t>((keys[i] << 16) | tok) << 32) | payload(tok);
+                              (static_cast<uint64_t>((keys[i] << 16) | tok) << 32) | payload(tok, i);
                         });
   for (uint32_t i = n_take + lane; i < cand_stride; i += kWave) dst[i] = kEmptyCand64;
 }

@@ -311,9 +311,25 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
       keys[p8 * 8 + 2 * i + 1] = hi == 0xffffu ? kInvalidKey : hi;
     }
   }
+  // One pass: the K rows of the lane's eight tokens are fetched with the keys (two 128-bit reads), so
+  // that no emitted candidate waits for an LDS round trip of its own.  With more passes the 16 or 32
+  // extra registers cost more than the waits (measured at 131072 tokens), and the rows are read as
+  // they are needed.
+  constexpr bool kRowsAhead = kItems == 8;
+  uint32_t krows[kRowsAhead ? kItems : 1];
+  if (kRowsAhead) {
+#pragma unroll
+    for (int p4 = 0; p4 < kItems / 4; ++p4) {
+      const uint4 v = *reinterpret_cast<const uint4*>(&sh.krow[lane * kItems + p4 * 4]);
+      krows[p4 * 4] = v.x;
+      krows[p4 * 4 + 1] = v.y;
+      krows[p4 * 4 + 2] = v.z;
+      krows[p4 * 4 + 3] = v.w;
+    }
+  }
   chunk_select_emit<kItems>(keys, min(kChunk, n - chunk_base), k, cand_stride, dst, hrow,
-                            sh.hist[wave], [&](uint32_t tok) __attribute__((always_inline)) {
-                              return sh.krow[tok];
+                            sh.hist[wave], [&](uint32_t tok, int i) __attribute__((always_inline)) {
+                              return kRowsAhead ? krows[kRowsAhead ? i : 0] : sh.krow[tok];
                             });
 }
 

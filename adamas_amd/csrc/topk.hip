@@ -324,7 +324,7 @@ __global__ __launch_bounds__(kIntWaves* kWave) void select_chunks_int_kernel(
   const int32_t* irow =
       a.in_idx ? a.in_idx + static_cast<int64_t>(row) * a.in_idx_stride : nullptr;
   chunk_select_emit<kItems>(keys, min(kChunk, n - chunk_base), a.k, cand_stride, dst, hrow,
-                            hist_lds[wave], [&](uint32_t item) __attribute__((always_inline)) {
+                            hist_lds[wave], [&](uint32_t item, int) __attribute__((always_inline)) {
                               const uint32_t e = chunk_base + item;
                               return irow ? static_cast<uint32_t>(irow[e]) : e;
                             });
