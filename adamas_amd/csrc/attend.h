@@ -116,24 +116,35 @@ struct SoftmaxState {
 //                       translated through the page table;
 //   kRowIndex == true : pos_of gives the K row index page*row_mult + slot directly (negative =
 //                       skip), no table access.
-//   kAllValid (with kRowIndex): every list entry is a valid row index; slots past row_end then load
-//                       the last row of the list again (its weight is zero) instead of branching
-//                       around the loads.
-template <int kGroups, int kTile, bool kRowIndex = false, bool kBf16 = false, bool kAllValid = false,
+//   kLoadAlways: no branch around the loads.  A slot past row_end reads the last list entry again
+//                       and an unused entry reads row 0 of the pool (kRowIndex) or token 0 of the
+//                       sequence, all with weight zero: the loads cost less than the branches and
+//                       the zeroed registers they replace.  A sequence without tokens is left
+//                       before the first load.
+template <int kGroups, int kTile, bool kRowIndex = false, bool kBf16 = false, bool kLoadAlways = false,
           typename PosFn>
 __device__ __forceinline__ void attend_rows(const HeadKV& kv, const float (&qf)[8], uint32_t g,
                                             uint32_t row_begin, uint32_t row_end, PosFn&& pos_of,
                                             SoftmaxState& st) {
-  static_assert(!kAllValid || kRowIndex, "kAllValid is for lists of row indices");
+  if (kLoadAlways && !kRowIndex && kv.seq_len <= 0) return;  // no token a clamped position could name
   for (uint32_t base = row_begin; base < row_end; base += kGroups * kTile) {
     uint4 kr[kTile], vr[kTile];
     bool valid[kTile];
 #pragma unroll
     for (int i = 0; i < kTile; ++i) {
       const uint32_t r = base + i * kGroups + g;
-      if (kAllValid) {
-        valid[i] = r < row_end;
-        const uint32_t row = static_cast<uint32_t>(pos_of(min(r, row_end - 1u)));
+      if (kLoadAlways) {
+        const int32_t pos = pos_of(min(r, row_end - 1u));
+        uint32_t row;
+        if (kRowIndex) {
+          valid[i] = r < row_end && pos >= 0;
+          row = static_cast<uint32_t>(max(pos, 0));
+        } else {
+          valid[i] = r < row_end && pos >= 0 && pos < kv.seq_len;
+          const uint32_t pc = static_cast<uint32_t>(min(max(pos, 0), kv.seq_len - 1));
+          const uint32_t lp = pc / kv.page_size;
+          row = static_cast<uint32_t>(kv.table[lp]) * kv.row_mult + (pc - lp * kv.page_size);
+        }
         const __half* kp = kv.kv_data + static_cast<size_t>(row) * kv.tok_stride + kv.head_off;
         kr[i] = *reinterpret_cast<const uint4*>(kp);
         vr[i] = *reinterpret_cast<const uint4*>(kp + kv.v_delta);
