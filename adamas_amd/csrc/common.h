@@ -89,6 +89,14 @@ __device__ __forceinline__ void store_elem(__half* p, float x) {
   *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(elem_bits<kBf16>(x));
 }
 
+// Key/value head of a query head, head / group with group = num_heads / num_kv_heads, without a
+// division in the kernel: the host passes the 16-bit reciprocal of the group size.  Exact while
+// head * group < 65536 (the host checks num_heads * group).
+inline uint32_t group_inv16(uint32_t group) { return (65536u + group - 1u) / group; }
+__device__ __forceinline__ uint32_t kv_head_of(uint32_t head, uint32_t inv16) {
+  return (head * inv16) >> 16;
+}
+
 // Physical location of logical token t of a sequence whose page table starts at `table`.
 template <typename T>
 __device__ __forceinline__ T token_slot(const int32_t* __restrict__ table, uint32_t t,

@@ -103,9 +103,10 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ seq_lens, uint64_t* __restrict__ cand,
     unsigned char* __restrict__ hist_out, uint32_t hist_stride, uint32_t k, uint32_t cand_stride,
-    uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size_rt, uint32_t table_stride,
-    uint32_t rows_per_page, uint16_t* __restrict__ dist_out = nullptr, int64_t dist_stride = 0,
-    uint32_t* __restrict__ rowmap_out = nullptr, QkvSource src = QkvSource()) {
+    uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_inv16, uint32_t page_size_rt,
+    uint32_t table_stride, uint32_t rows_per_page, uint16_t* __restrict__ dist_out = nullptr,
+    int64_t dist_stride = 0, uint32_t* __restrict__ rowmap_out = nullptr,
+    QkvSource src = QkvSource()) {
   static_assert(!kHist || kPasses == 1, "the histogram mode works on 512-token chunks");
   constexpr uint32_t kChunk = kFusedBlock * kPasses;  // tokens per workgroup
   constexpr int kItems = 8 * kPasses;                 // tokens per lane in the selection phase
@@ -200,9 +201,10 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
 
     // grouped-query attention: query head h scores the codes of key head h / group; the lanes of a
     // group load the same bytes, and the workgroups of a group read the same rows through L2
-    const size_t row_bytes = static_cast<size_t>(num_kv_heads) * 32u;
-    const unsigned char* lane_base =
-        code_data + (head / (num_heads / num_kv_heads)) * 32u + half * 16u;
+    // (32-bit operands: the byte offset of a token is then one 32 x 32 -> 64 bit multiply-add per
+    // load, and the key/value head comes from the reciprocal of the group size, not a division)
+    const uint32_t row_bytes = num_kv_heads * 32u;
+    const unsigned char* lane_base = code_data + kv_head_of(head, kv_inv16) * 32u + half * 16u;
 
     // issues the 16 loads of pass `pass` (tokens pass*512 + wave*64 .. +63 of the chunk); tokens past
     // the end of the sequence read some valid slot and are masked when the distances are stored
@@ -221,7 +223,9 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
           in_page = t % page_size;
         }
         kw[j] = *reinterpret_cast<const uint4*>(
-            lane_base + (static_cast<size_t>(page) * page_size + in_page) * row_bytes);
+            lane_base + static_cast<size_t>(page * page_size + in_page) * row_bytes);
+        // (written between the loads on purpose: with the 16 loads of a wave back to back the
+        // launch is 0.1 us slower from HBM, although 0.2 us faster from the Infinity Cache)
         if ((static_cast<uint32_t>(lane) % kTokLanes) == 0)
           sh.krow[tok0 + j * kLoadTokens + sub] = page * rows_per_page + in_page;
       }
@@ -355,8 +359,9 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     const int32_t* __restrict__ seq_lens, const uint64_t* __restrict__ cand,
     const unsigned char* __restrict__ hist, uint32_t hist_stride, uint32_t n_chunks,
     uint32_t chunk_tokens, uint32_t k, uint32_t cand_stride, __half* __restrict__ out,
-    int32_t* __restrict__ sel_out, uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size,
-    float scale_log2, uint32_t table_stride, QkvSource src = QkvSource(),
+    int32_t* __restrict__ sel_out, uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_group,
+    uint32_t kv_inv16, uint32_t page_size, float scale_log2, uint32_t table_stride,
+    QkvSource src = QkvSource(),
     __half* kv_append = nullptr, uint16_t* code_data = nullptr) {
   static_assert(!kFromQkv || (!kBf16 && !kHnd), "the fused projection is fp16 over NHD pages");
   static_assert(kAttThreads == kFinalThreads, "final_select runs on the whole workgroup");
@@ -399,9 +404,9 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   // value row (lane l = channels 2l and 2l+1).  The loads are issued here and used inside the
   // selection, once its own loads are under way; the results go to the other waves through LDS.
   WaveRopeLoads row_now = {};
-  const uint32_t kv_head_now = head / (num_heads / num_kv_heads);
+  const uint32_t kv_head_now = kv_head_of(head, kv_inv16);  // kv_group = num_heads / num_kv_heads
   // the waves that append the new token of this head's key/value head (one workgroup per key/value head)
-  const bool appends = kFromQkv && head % (num_heads / num_kv_heads) == 0;
+  const bool appends = kFromQkv && kv_head_now * kv_group == head;
   uint32_t kcode_word = 0, kpacked = 0;  // wave 1: code word and fp16 pair of the rotated new key
   if (kFromQkv) {
     if (wave < 3) {
@@ -491,7 +496,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   HeadKV kv;
   kv.kv_data = kv_data;
   kv.table = nullptr;  // rows are K row indices already
-  set_kv_layout_static<kHnd>(kv, head / (num_heads / num_kv_heads), c16, num_kv_heads, page_size);
+  set_kv_layout_static<kHnd>(kv, kv_head_now, c16, num_kv_heads, page_size);
   kv.seq_len = seq_len;
   SoftmaxState st;
   attend_rows<32, 4, true, kBf16, true>(kv, qf, g, 0u, kFromQkv ? n_take : n_take + 1u,
@@ -590,6 +595,8 @@ static int step_candidates_impl(const void* q_code, const void* code_data,
     return ADAMAS_E_BADARG;
   if (num_heads == 0 || num_heads % 32 != 0 || batch > 65535) return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
+  // the kernels take head / group from a 16-bit reciprocal (kv_head_of)
+  if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(workspace) & 255) return ADAMAS_E_ALIGN;
   if ((reinterpret_cast<uintptr_t>(q_code) | reinterpret_cast<uintptr_t>(code_data)) & 15)
     return ADAMAS_E_ALIGN;
@@ -608,7 +615,8 @@ static int step_candidates_impl(const void* q_code, const void* code_data,
                      static_cast<const uint16_t*>(q_code),                                    \
                      static_cast<const unsigned char*>(code_data), page_indices, page_indptr, \
                      seq_lens, cand, hist, w.hist_stride, budget - 1, w.cand_stride,          \
-                     num_heads, num_kv_heads, page_size, page_table_stride,                   \
+                     num_heads, num_kv_heads, group_inv16(num_heads / num_kv_heads),         \
+                     page_size, page_table_stride,                                            \
                      rows_per_page_of(flags, page_size, num_kv_heads),                        \
                      static_cast<uint16_t*>(nullptr), static_cast<int64_t>(0),                \
                      static_cast<uint32_t*>(nullptr), qsrc ? *qsrc : QkvSource())
@@ -693,6 +701,8 @@ static int step_attend_impl(const void* q, void* kv_data, const int32_t* page_in
   if (head_dim != kHeadDim || num_heads == 0 || num_heads % 32 != 0 || batch > 65535)
     return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
+  // the kernels take head / group from a 16-bit reciprocal (kv_head_of)
+  if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(workspace) & 255) return ADAMAS_E_ALIGN;
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kv_data)) & 15)
     return ADAMAS_E_ALIGN;
@@ -708,7 +718,8 @@ static int step_attend_impl(const void* q, void* kv_data, const int32_t* page_in
                      reinterpret_cast<const uint64_t*>(ws + w.cand_off),                        \
                      reinterpret_cast<const unsigned char*>(ws + w.hist_off), w.hist_stride,    \
                      w.cand_chunks, w.chunk_tokens, budget - 1, w.cand_stride,                  \
-                     static_cast<__half*>(out), sel_out, num_heads, num_kv_heads, page_size,    \
+                     static_cast<__half*>(out), sel_out, num_heads, num_kv_heads,               \
+                     num_heads / num_kv_heads, group_inv16(num_heads / num_kv_heads), page_size, \
                      sm_scale * 1.4426950408889634f, page_table_stride,                          \
                      qsrc ? *qsrc : QkvSource(), static_cast<__half*>(kv_data),                  \
                      static_cast<uint16_t*>(code_data))
@@ -782,6 +793,8 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
     return ADAMAS_E_BADARG;
   if (head_dim != kHeadDim || num_heads == 0 || num_heads % 32 != 0) return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
+  // the kernels take head / group from a 16-bit reciprocal (kv_head_of)
+  if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;
   if (batch > 65535) return ADAMAS_E_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(workspace) & 255) return ADAMAS_E_ALIGN;
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(q_code) |
@@ -823,7 +836,8 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
                      static_cast<const uint16_t*>(q_code),                                      \
                      static_cast<const unsigned char*>(code_data), page_indices, page_indptr,   \
                      seq_lens, static_cast<uint64_t*>(nullptr), hist, w.hist_stride, n_sel, 0u, \
-                     num_heads, num_kv_heads, page_size, page_table_stride,                     \
+                     num_heads, num_kv_heads, group_inv16(num_heads / num_kv_heads),           \
+                     page_size, page_table_stride,                                              \
                      rows_per_page_of(flags, page_size, num_kv_heads), dist,                    \
                      static_cast<int64_t>(w.dist_stride), rowmap)
 #define ADAMAS_LAUNCH_ESTHIST(PG)        \
