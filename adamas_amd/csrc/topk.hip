@@ -69,8 +69,30 @@ __device__ __forceinline__ uint32_t row_length(const SelectArgs& a, uint32_t row
 }
 
 // keys of items e0..e0+7 of a row of values (n = row length)
+// kPadded: the row is backed up to a multiple of 8 elements (and vec_ok holds), so the group that
+// holds the end of the row is read with one 128-bit load as well and masked afterwards.
+template <bool kPadded = false>
 __device__ __forceinline__ void load_value_keys(const uint16_t* vrow, uint32_t e0, uint32_t n,
                                                 bool vec_ok, uint32_t key_mode, uint32_t* keys) {
+  if (kPadded) {
+    if (e0 < n) {
+      const uint4 v = *reinterpret_cast<const uint4*>(vrow + e0);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        keys[2 * i] = make_key(w[i] & 0xffffu, key_mode);
+        keys[2 * i + 1] = make_key(w[i] >> 16, key_mode);
+      }
+      if (e0 + 8 > n) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) keys[r] = (e0 + r < n) ? keys[r] : kInvalidKey;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) keys[r] = kInvalidKey;
+    }
+    return;
+  }
   if (vec_ok && e0 + 8 <= n) {
     const uint4 v = *reinterpret_cast<const uint4*>(vrow + e0);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -561,8 +583,15 @@ struct HistEmitShared {
 };
 
 // chunks_per_slab: histogram rows per 4096 keys (4 for chunks of 1024 keys, 8 for chunks of 512).
+// kKeyMode >= 0: the key format is known at compile time and the rows are read with 128-bit loads
+// (the caller has checked their alignment); -1: both are taken from the arguments.  The instances
+// with a fixed format leave out the element-wise loads and the other formats' conversions, which
+// are most of the code of the general one.  kPadded: see load_value_keys.
+template <int kKeyMode, bool kPadded = false>
 __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
     SelectArgs a, const uint16_t* __restrict__ hist, uint32_t n_chunks, uint32_t chunks_per_slab) {
+  const uint32_t key_mode = kKeyMode >= 0 ? static_cast<uint32_t>(kKeyMode) : a.key_mode;
+  const bool vec_ok = kKeyMode >= 0 || a.vec_ok != 0;
   constexpr int kWaves = kEmitThreads / kWave;
   __shared__ HistEmitShared sh;
   const uint32_t row = blockIdx.x, slab = blockIdx.y;
@@ -583,7 +612,7 @@ __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
   uint32_t keys[kEmitItems];
 #pragma unroll
   for (int j = 0; j < kEmitItems / 8; ++j)
-    load_value_keys(vrow, e0 + j * 8, n, a.vec_ok != 0, a.key_mode, &keys[j * 8]);
+    load_value_keys<kPadded>(vrow, e0 + j * 8, n, vec_ok, key_mode, &keys[j * 8]);
 
   // the K row indices of the same 16 tokens, when asked for (16-byte aligned: rows of the map are)
   int32_t* rdst = a.out_rows ? a.out_rows + static_cast<int64_t>(row) * a.out_stride : nullptr;
@@ -706,7 +735,7 @@ __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
                               if (rdst) rdst[pos] = static_cast<int32_t>(trow[i]);
                               if (vdst)
                                 vdst[pos] =
-                                    static_cast<uint16_t>(raw_of_key(keys[i], a.key_mode));
+                                    static_cast<uint16_t>(raw_of_key(keys[i], key_mode));
                             });
   if (slab == 0) {
     for (uint32_t i = plan.n_take + tid; i < k; i += kEmitThreads) {
@@ -744,8 +773,14 @@ int launch_hist_select(const uint16_t* dist, int64_t row_stride, uint32_t n_max,
   a.rowmap = rowmap;
   a.rowmap_stride = rowmap_stride;
   a.out_rows = out_rows;
-  hipLaunchKernelGGL(select_hist_emit_kernel, dim3(num_rows, ceil_div(n_max, kEmitSlab)),
-                     dim3(kEmitThreads), 0, stream, a, hist, n_chunks, kEmitSlab / chunk_keys);
+  // the distance rows of the step's workspace are aligned and padded to a multiple of 8 elements
+  if (a.vec_ok && row_stride >= static_cast<int64_t>((n_max + 7) / 8 * 8))
+    hipLaunchKernelGGL((select_hist_emit_kernel<ADAMAS_KEY_U16_INT, true>),
+                       dim3(num_rows, ceil_div(n_max, kEmitSlab)), dim3(kEmitThreads), 0, stream, a,
+                       hist, n_chunks, kEmitSlab / chunk_keys);
+  else
+    hipLaunchKernelGGL(select_hist_emit_kernel<-1>, dim3(num_rows, ceil_div(n_max, kEmitSlab)),
+                       dim3(kEmitThreads), 0, stream, a, hist, n_chunks, kEmitSlab / chunk_keys);
   ADAMAS_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
@@ -854,8 +889,16 @@ extern "C" int adamas_topk(const void* values, int64_t row_stride, uint32_t n_ma
                        dim3(kHistWaves * kWave), 0, s, a, hist, n_chunks);
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
     if (n_max <= kEmitMaxRowLen) {
-      hipLaunchKernelGGL(select_hist_emit_kernel, dim3(num_rows, ceil_div(n_max, kEmitSlab)),
-                         dim3(kEmitThreads), 0, s, a, hist, n_chunks, kEmitSlab / kHistChunk);
+      const dim3 egrid(num_rows, ceil_div(n_max, kEmitSlab));
+      if (a.vec_ok && key_mode == ADAMAS_KEY_FP16_INT)
+        hipLaunchKernelGGL(select_hist_emit_kernel<ADAMAS_KEY_FP16_INT>, egrid, dim3(kEmitThreads),
+                           0, s, a, hist, n_chunks, kEmitSlab / kHistChunk);
+      else if (a.vec_ok && key_mode == ADAMAS_KEY_U16_INT)
+        hipLaunchKernelGGL(select_hist_emit_kernel<ADAMAS_KEY_U16_INT>, egrid, dim3(kEmitThreads),
+                           0, s, a, hist, n_chunks, kEmitSlab / kHistChunk);
+      else
+        hipLaunchKernelGGL(select_hist_emit_kernel<-1>, egrid, dim3(kEmitThreads), 0, s, a, hist,
+                           n_chunks, kEmitSlab / kHistChunk);
     } else {
       hipLaunchKernelGGL(select_hist_final_kernel, dim3(num_rows), dim3(1024), 0, s, a, hist,
                          n_chunks);
