@@ -316,10 +316,13 @@ static IntLayout int_layout(uint32_t num_rows, uint32_t n_max, uint32_t k) {
 }
 
 // level 1: grid (ceil(n_chunks / 8), rows), 512 threads; wave w takes chunk blockIdx.x * 8 + w
-template <int kItems>
+// kKeyMode: as for select_hist_emit_kernel (>= 0: format fixed at compile time, aligned rows)
+template <int kItems, int kKeyMode>
 __global__ __launch_bounds__(kIntWaves* kWave) void select_chunks_int_kernel(
     SelectArgs a, uint64_t* __restrict__ cand, unsigned char* __restrict__ hist, uint32_t n_chunks,
     uint32_t cand_stride) {
+  const uint32_t key_mode = kKeyMode >= 0 ? static_cast<uint32_t>(kKeyMode) : a.key_mode;
+  const bool vec_ok = kKeyMode >= 0 || a.vec_ok != 0;
   __shared__ alignas(16) uint32_t hist_lds[kIntWaves][kHistBins / 2];
   const int lane = lane_id();
   const int wave = wave_id_uniform();
@@ -342,7 +345,7 @@ __global__ __launch_bounds__(kIntWaves* kWave) void select_chunks_int_kernel(
 #pragma unroll
   for (int j = 0; j < kItems / 8; ++j)
     load_value_keys(vrow, chunk_base + static_cast<uint32_t>(lane) * kItems + j * 8, n,
-                    a.vec_ok != 0, a.key_mode, &keys[j * 8]);
+                    vec_ok, key_mode, &keys[j * 8]);
   const int32_t* irow =
       a.in_idx ? a.in_idx + static_cast<int64_t>(row) * a.in_idx_stride : nullptr;
   chunk_select_emit<kItems>(keys, min(kChunk, n - chunk_base), a.k, cand_stride, dst, hrow,
@@ -399,8 +402,12 @@ constexpr int kHistItems = 16;                        // keys per lane
 constexpr uint32_t kHistChunk = kWave * kHistItems;   // 1024 keys per chunk
 constexpr uint32_t kHistRowBytes = kHistBins * 2;     // one chunk's counts
 
+// kKeyMode: as for select_hist_emit_kernel (>= 0: format fixed at compile time, aligned rows)
+template <int kKeyMode>
 __global__ __launch_bounds__(kHistWaves* kWave) void hist_chunks_int_kernel(
     SelectArgs a, uint16_t* __restrict__ hist, uint32_t n_chunks) {
+  const uint32_t key_mode = kKeyMode >= 0 ? static_cast<uint32_t>(kKeyMode) : a.key_mode;
+  const bool vec_ok = kKeyMode >= 0 || a.vec_ok != 0;
   __shared__ uint32_t h[kHistWaves][kHistBins / 2];  // two 16-bit bins per word
   const int lane = lane_id();
   const int wave = wave_id_uniform();
@@ -417,7 +424,7 @@ __global__ __launch_bounds__(kHistWaves* kWave) void hist_chunks_int_kernel(
 #pragma unroll
     for (int j = 0; j < kHistItems / 8; ++j)
       load_value_keys(vrow, chunk_base + static_cast<uint32_t>(lane) * kHistItems + j * 8, n,
-                      a.vec_ok != 0, a.key_mode, &keys[j * 8]);
+                      vec_ok, key_mode, &keys[j * 8]);
 #pragma unroll
     for (int i = 0; i < kHistItems; ++i)  // a bin holds at most 1024 entries: no carry into its neighbour
       if (keys[i] != kInvalidKey) atomicAdd(&hw[keys[i] >> 1], 1u << (16 * (keys[i] & 1u)));
@@ -851,16 +858,27 @@ extern "C" int adamas_topk(const void* values, int64_t row_stride, uint32_t n_ma
     uint64_t* cand = static_cast<uint64_t*>(workspace);
     unsigned char* hist = static_cast<unsigned char*>(workspace) + il.cand_bytes;
     const dim3 grid1(ceil_div(il.n_chunks, kIntWaves), num_rows);
+    // the instance with the key format compiled in, where the rows allow 128-bit loads
+#define ADAMAS_LAUNCH_CHUNKS_INT(ITEMS, MODE)                                                    \
+  hipLaunchKernelGGL((select_chunks_int_kernel<ITEMS, MODE>), grid1, dim3(kIntWaves * kWave), 0, \
+                     s, a, cand, hist, il.n_chunks, il.cand_stride)
+#define ADAMAS_LAUNCH_CHUNKS_INT_MODE(ITEMS)                          \
+  if (a.vec_ok && key_mode == ADAMAS_KEY_FP16_INT) {                  \
+    ADAMAS_LAUNCH_CHUNKS_INT(ITEMS, static_cast<int>(ADAMAS_KEY_FP16_INT)); \
+  } else if (a.vec_ok && key_mode == ADAMAS_KEY_U16_INT) {            \
+    ADAMAS_LAUNCH_CHUNKS_INT(ITEMS, static_cast<int>(ADAMAS_KEY_U16_INT));  \
+  } else {                                                            \
+    ADAMAS_LAUNCH_CHUNKS_INT(ITEMS, -1);                              \
+  }
     if (il.items == 8) {
-      hipLaunchKernelGGL(select_chunks_int_kernel<8>, grid1, dim3(kIntWaves * kWave), 0, s, a, cand,
-                         hist, il.n_chunks, il.cand_stride);
+      ADAMAS_LAUNCH_CHUNKS_INT_MODE(8)
     } else if (il.items == 16) {
-      hipLaunchKernelGGL(select_chunks_int_kernel<16>, grid1, dim3(kIntWaves * kWave), 0, s, a, cand,
-                         hist, il.n_chunks, il.cand_stride);
+      ADAMAS_LAUNCH_CHUNKS_INT_MODE(16)
     } else {
-      hipLaunchKernelGGL(select_chunks_int_kernel<32>, grid1, dim3(kIntWaves * kWave), 0, s, a, cand,
-                         hist, il.n_chunks, il.cand_stride);
+      ADAMAS_LAUNCH_CHUNKS_INT_MODE(32)
     }
+#undef ADAMAS_LAUNCH_CHUNKS_INT_MODE
+#undef ADAMAS_LAUNCH_CHUNKS_INT
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
     const uint64_t slots = static_cast<uint64_t>(il.n_chunks) * il.cand_stride;
 #define ADAMAS_LAUNCH_FINAL(G)                                                                      \
@@ -885,8 +903,16 @@ extern "C" int adamas_topk(const void* values, int64_t row_stride, uint32_t n_ma
       (reinterpret_cast<uintptr_t>(workspace) & 255) == 0) {
     const uint32_t n_chunks = ceil_div(n_max, kHistChunk);
     uint16_t* hist = static_cast<uint16_t*>(workspace);
-    hipLaunchKernelGGL(hist_chunks_int_kernel, dim3(ceil_div(n_chunks, kHistWaves), num_rows),
-                       dim3(kHistWaves * kWave), 0, s, a, hist, n_chunks);
+    const dim3 hgrid(ceil_div(n_chunks, kHistWaves), num_rows);
+    if (a.vec_ok && key_mode == ADAMAS_KEY_FP16_INT)
+      hipLaunchKernelGGL(hist_chunks_int_kernel<static_cast<int>(ADAMAS_KEY_FP16_INT)>, hgrid,
+                         dim3(kHistWaves * kWave), 0, s, a, hist, n_chunks);
+    else if (a.vec_ok && key_mode == ADAMAS_KEY_U16_INT)
+      hipLaunchKernelGGL(hist_chunks_int_kernel<static_cast<int>(ADAMAS_KEY_U16_INT)>, hgrid,
+                         dim3(kHistWaves * kWave), 0, s, a, hist, n_chunks);
+    else
+      hipLaunchKernelGGL(hist_chunks_int_kernel<-1>, hgrid, dim3(kHistWaves * kWave), 0, s, a, hist,
+                         n_chunks);
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
     if (n_max <= kEmitMaxRowLen) {
       const dim3 egrid(num_rows, ceil_div(n_max, kEmitSlab));
