@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void estimate_kernel(
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ seq_lens, uint16_t* __restrict__ out, int64_t out_bs,
     int64_t out_hs, uint32_t out_format, uint32_t num_heads, uint32_t num_kv_heads,
-    uint32_t page_size_rt, uint32_t vec_ok) {
+    uint32_t kv_inv16, uint32_t page_size_rt, uint32_t vec_ok) {
   const uint32_t page_size = kPage ? static_cast<uint32_t>(kPage) : page_size_rt;
   const uint32_t b = blockIdx.y;
   const uint32_t seg = blockIdx.z;  // group of 32 heads
@@ -48,26 +48,27 @@ __global__ __launch_bounds__(256) void estimate_kernel(
   const int32_t* table = page_indices + page_indptr[b];
   // grouped-query attention: query head h reads the codes of key head h / (num_heads / num_kv_heads);
   // lanes of one group then load the same bytes (merged by the memory pipeline)
-  const uint32_t kv_head = head / (num_heads / num_kv_heads);
-  const size_t row_bytes = static_cast<size_t>(num_kv_heads) * 32u;
+  // (from the reciprocal of the group size; 32-bit strides: one multiply-add per load address)
+  const uint32_t kv_head = kv_head_of(head, kv_inv16);
+  const uint32_t row_bytes = num_kv_heads * 32u;
   const unsigned char* lane_base = code_data + kv_head * 32u + half * 16u;
 
   uint4 kw[kTokPerWave];
   const uint32_t last = static_cast<uint32_t>(n) - 1u;
   if (kPage == 16) {
     // t0 is a multiple of 16: all 16 tokens sit in one page
-    const size_t slot0 = static_cast<size_t>(table[t0 >> 4]) * 16u;
+    const uint32_t slot0 = static_cast<uint32_t>(table[t0 >> 4]) * 16u;
 #pragma unroll
     for (int j = 0; j < kTokPerWave; ++j) {
       uint32_t s = min(t0 + j, last) - t0;
-      kw[j] = *reinterpret_cast<const uint4*>(lane_base + (slot0 + s) * row_bytes);
+      kw[j] = *reinterpret_cast<const uint4*>(lane_base + static_cast<size_t>(slot0 + s) * row_bytes);
     }
   } else {
 #pragma unroll
     for (int j = 0; j < kTokPerWave; ++j) {
       uint32_t t = min(t0 + j, last);
-      size_t slot = token_slot<size_t>(table, t, page_size);
-      kw[j] = *reinterpret_cast<const uint4*>(lane_base + slot * row_bytes);
+      const uint32_t slot = token_slot<uint32_t>(table, t, page_size);
+      kw[j] = *reinterpret_cast<const uint4*>(lane_base + static_cast<size_t>(slot) * row_bytes);
     }
   }
 
@@ -152,6 +153,8 @@ extern "C" int adamas_estimate(const void* q_code, const void* code_data,
     return ADAMAS_E_BADARG;
   if (num_heads == 0 || num_heads % 32 != 0) return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
+  // the kernel takes head / group from a 16-bit reciprocal (kv_head_of)
+  if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;
   if (out_format != ADAMAS_DIST_FP16 && out_format != ADAMAS_DIST_U16) return ADAMAS_E_BADARG;
   if ((reinterpret_cast<uintptr_t>(q_code) | reinterpret_cast<uintptr_t>(code_data)) & 15)
     return ADAMAS_E_ALIGN;
@@ -170,7 +173,8 @@ extern "C" int adamas_estimate(const void* q_code, const void* code_data,
                      static_cast<const uint16_t*>(q_code),                                     \
                      static_cast<const unsigned char*>(code_data), page_indices, page_indptr,  \
                      seq_lens, static_cast<uint16_t*>(out), out_batch_stride, out_head_stride, \
-                     out_format, num_heads, num_kv_heads, page_size, vec_ok)
+                     out_format, num_heads, num_kv_heads,                                       \
+                     group_inv16(num_heads / num_kv_heads), page_size, vec_ok)
   if (page_size == 16) {
     ADAMAS_LAUNCH_ESTIMATE(16);
   } else if (page_size == 1) {
