@@ -17,6 +17,9 @@
 namespace adamas {
 
 constexpr int kHistBins = 512;                  // key values 0..511
+// LDS words of chunk_select_emit's histogram, per wave: one 32-bit counter per key value and, behind
+// them, a counter that takes the items that are no keys (padded to a multiple of 16 bytes)
+constexpr int kChunkHistWords = kHistBins + 4;
 constexpr uint64_t kEmptyCand64 = ~0ull;        // an unused candidate slot
 constexpr int kFinalThreads = 512;              // workgroup of final_select: one thread per bin
 constexpr int kFinalWaves = kFinalThreads / kWave;
@@ -87,13 +90,13 @@ __device__ __forceinline__ void raw_class_masks(const uint32_t (&keys)[kItems], 
 }
 
 // One wave: the k smallest of its 64 x kItems keys (lane l holds items kItems*l .. kItems*l + kItems-1,
-// kInvalidKey = no item; n_valid = number of items).  dst: the chunk's candidate list (cand_stride
+// any value above 511, e.g. kInvalidKey, = no item; n_valid = number of items).  dst: the chunk's candidate list (cand_stride
 // slots, unused ones are filled with kEmptyCand64); hrow: this lane's 8 bytes of the chunk's
-// histogram row; hist_lds: 256 words of LDS owned by this wave, 16-byte aligned; payload(item, i) -> 32
+// histogram row; hist_lds: kChunkHistWords words of LDS owned by this wave, 16-byte aligned; payload(item, i) -> 32
 // bits stored with the candidate (evaluated for selected items only; i = item - kItems * lane is a
 // constant at every call, so a caller can keep its payloads in registers).
 // The threshold is read off a histogram instead of being searched for: every lane counts its keys
-// into 512 bins of 16-bit counters in LDS, a prefix sum over the bins (8 bins per lane, DPP scan
+// into 512 counters in LDS, a prefix sum over the bins (8 bins per lane, DPP scan
 // across the lanes) finds the bin that holds the k-th smallest key, and the histogram of the
 // candidates follows from the same counts (bins below the threshold whole, the threshold bin up to
 // the tie quota).  Measured against a 7-round bisection on byte-packed keys (one add + and + popcount
@@ -106,14 +109,18 @@ __device__ __forceinline__ void chunk_select_emit(const uint32_t (&keys)[kItems]
                                                        uint2* hrow, uint32_t* hist_lds,
                                                        Payload&& payload) {
   const int lane = lane_id();
-  *reinterpret_cast<uint4*>(&hist_lds[4 * lane]) = make_uint4(0u, 0u, 0u, 0u);
+  *reinterpret_cast<uint4*>(&hist_lds[8 * lane]) = make_uint4(0u, 0u, 0u, 0u);
+  *reinterpret_cast<uint4*>(&hist_lds[8 * lane + 4]) = make_uint4(0u, 0u, 0u, 0u);
+  // One 32-bit counter per key value, and no branch: an item that is no key (any value above 511) counts
+  // into the word behind the last bin, which nobody reads.  (Packing two 16-bit bins into a word
+  // and skipping the invalid items cost seven more instructions per item.)
 #pragma unroll
-  for (int i = 0; i < kItems; ++i)  // a bin holds at most 64 * kItems <= 2048 keys: no carry
-    if (keys[i] != kInvalidKey) atomicAdd(&hist_lds[keys[i] >> 1], 1u << (16 * (keys[i] & 1u)));
+  for (int i = 0; i < kItems; ++i)
+    atomicAdd(&hist_lds[min(keys[i], static_cast<uint32_t>(kHistBins))], 1u);
   // the LDS operations of one wave are carried out in order: the counts are complete here
-  const uint4 hv = *reinterpret_cast<const uint4*>(&hist_lds[4 * lane]);
-  const uint32_t c[8] = {hv.x & 0xffffu, hv.x >> 16, hv.y & 0xffffu, hv.y >> 16,
-                         hv.z & 0xffffu, hv.z >> 16, hv.w & 0xffffu, hv.w >> 16};
+  const uint4 hv0 = *reinterpret_cast<const uint4*>(&hist_lds[8 * lane]);
+  const uint4 hv1 = *reinterpret_cast<const uint4*>(&hist_lds[8 * lane + 4]);
+  const uint32_t c[8] = {hv0.x, hv0.y, hv0.z, hv0.w, hv1.x, hv1.y, hv1.z, hv1.w};
   uint32_t lane_sum = 0;
 #pragma unroll
   for (int j = 0; j < 8; ++j) lane_sum += c[j];

@@ -44,9 +44,10 @@ template <int kPasses, int kHeads>
 struct EstimateSelectShared {
   alignas(16) uint16_t dist[kHeads][kFusedBlock * kPasses + kDistRowPad];  // 0xFFFF = no token
   uint32_t krow[kFusedBlock * kPasses];       // K row index (page * rows per page + slot) of every token
-  // tokens per distance value of one head, two 16-bit bins per word: read off for the chunk's
-  // threshold (selection) or written out (histogram mode); rows are read with 128-bit accesses
-  alignas(16) uint32_t hist[kHeads][kHistBins / 2];
+  // tokens per distance value of one head: one word per value, read off for the chunk's threshold
+  // (selection), or two 16-bit bins per word in the first 256 words, written out as they are
+  // (histogram mode); rows are read with 128-bit accesses
+  alignas(16) uint32_t hist[kHeads][kChunkHistWords];
   alignas(16) uint16_t qcode[kHeads][kCodeWords];  // query codes made in the kernel (kFromQkv)
 };
 
@@ -310,9 +311,9 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const uint32_t lo = w[i] & 0xffffu, hi = w[i] >> 16;
-      keys[p8 * 8 + 2 * i] = lo == 0xffffu ? kInvalidKey : lo;
-      keys[p8 * 8 + 2 * i + 1] = hi == 0xffffu ? kInvalidKey : hi;
+      // 0xffff (no token) stays as it is: above every threshold, and counted into the spare word
+      keys[p8 * 8 + 2 * i] = w[i] & 0xffffu;
+      keys[p8 * 8 + 2 * i + 1] = w[i] >> 16;
     }
   }
   // One pass: the K rows of the lane's eight tokens are fetched with the keys (two 128-bit reads), so

@@ -323,7 +323,7 @@ __global__ __launch_bounds__(kIntWaves* kWave) void select_chunks_int_kernel(
     uint32_t cand_stride) {
   const uint32_t key_mode = kKeyMode >= 0 ? static_cast<uint32_t>(kKeyMode) : a.key_mode;
   const bool vec_ok = kKeyMode >= 0 || a.vec_ok != 0;
-  __shared__ alignas(16) uint32_t hist_lds[kIntWaves][kHistBins / 2];
+  __shared__ alignas(16) uint32_t hist_lds[kIntWaves][kChunkHistWords];
   const int lane = lane_id();
   const int wave = wave_id_uniform();
   const uint32_t row = blockIdx.y;
