@@ -71,6 +71,28 @@ __device__ __forceinline__ void lane_emit(const uint32_t (&below)[kRegs],
   }
 }
 
+// The same without branches: emit is called for EVERY item, with position `dump` for the ones that
+// are not selected (the caller points that at a spare slot of its own for this lane).  Where emit is
+// a pair of LDS writes this costs fewer instructions than the compare-and-branch around each item.
+template <int kRegs, typename Emit>
+__device__ __forceinline__ void lane_emit_all(const uint32_t (&below)[kRegs],
+                                              const uint32_t (&equal)[kRegs], uint32_t n_below,
+                                              uint32_t quota, uint32_t pb, uint32_t pe,
+                                              uint32_t dump, Emit&& emit) {
+  pe += n_below;  // tied items go behind the ones below the threshold
+  const uint32_t pe_end = n_below + quota;
+#pragma unroll
+  for (int i = 0; i < 4 * kRegs; ++i) {
+    const uint32_t bit = 0x80u << (8 * (i & 3));
+    const bool is_b = (below[i >> 2] & bit) != 0;
+    const bool is_e = (equal[i >> 2] & bit) != 0;
+    const uint32_t pos = is_b ? pb : ((is_e && pe < pe_end) ? pe : dump);
+    emit(pos, i);
+    pb += is_b ? 1u : 0u;
+    pe += is_e ? 1u : 0u;
+  }
+}
+
 // class masks of kItems keys against a full-width threshold (bit 8r+7 of word j = item 4j+r)
 template <int kItems>
 __device__ __forceinline__ void raw_class_masks(const uint32_t (&keys)[kItems], uint32_t thr,
@@ -190,12 +212,15 @@ struct FinalSelectShared {
 // while_loading() is called once by every thread after the loads of the histogram rows and of the
 // candidates have been consumed and before the first barrier: work of the caller that depends on
 // loads it issued earlier costs no wait of its own there.
-template <int kGroups, typename Emit, typename WhileLoading>
+// kEmitAll: emit is called for every candidate slot, unselected ones with position dump_base + lane
+// (see lane_emit_all); the caller's arrays have 64 spare entries there.
+template <int kGroups, bool kEmitAll = false, typename Emit, typename WhileLoading>
 __device__ __forceinline__ uint32_t final_select(const uint64_t* __restrict__ crow, uint32_t n_slots,
                                                  const unsigned char* __restrict__ hist_rows,
                                                  uint32_t n_chunks, uint32_t k,
                                                  uint32_t cand_stride, FinalSelectShared& sh,
-                                                 Emit&& emit, WhileLoading&& while_loading) {
+                                                 Emit&& emit, WhileLoading&& while_loading,
+                                                 uint32_t dump_base = 0) {
   static_assert(kFinalThreads == kHistBins, "one thread per key value");
   constexpr int kItems = 8 * kGroups;
   constexpr int kAttThreads = kFinalThreads;
@@ -347,12 +372,16 @@ __device__ __forceinline__ uint32_t final_select(const uint64_t* __restrict__ cr
     // cand_stride is a multiple of 8: the 8 slots of a group belong to one chunk, slot0 / cand_stride
     // (left to the caller: a division per lane that only a caller who wants positions has to pay)
     const uint32_t slot0 = block_item_index<kItems>(wave, lane, j, 0);
-    lane_emit<2>(bj, ej, n_below, quota, base_b + (ex[j] & 0xffffu), base_e + (ex[j] >> 16),
-                 [&](uint32_t pos, int i) __attribute__((always_inline)) {
-                   const uint32_t tk = toks[j * 4 + (i >> 1)];
-                   emit(pos, slot0, (i & 1) ? (tk >> 16) : (tk & 0xffffu), keys[j * 8 + i],
-                        krow[j * 8 + i]);
-                 });
+    auto emit_item = [&](uint32_t pos, int i) __attribute__((always_inline)) {
+      const uint32_t tk = toks[j * 4 + (i >> 1)];
+      emit(pos, slot0, (i & 1) ? (tk >> 16) : (tk & 0xffffu), keys[j * 8 + i], krow[j * 8 + i]);
+    };
+    if (kEmitAll)
+      lane_emit_all<2>(bj, ej, n_below, quota, base_b + (ex[j] & 0xffffu),
+                       base_e + (ex[j] >> 16), dump_base + static_cast<uint32_t>(lane), emit_item);
+    else
+      lane_emit<2>(bj, ej, n_below, quota, base_b + (ex[j] & 0xffffu), base_e + (ex[j] >> 16),
+                   emit_item);
     base_b += tot[j] & 0xffffu;
     base_e += tot[j] >> 16;
   }

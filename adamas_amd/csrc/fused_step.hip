@@ -340,8 +340,10 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
 
 struct SelectAttendShared {
   MergeShared<32> merge;
-  int32_t rows[kFusedMaxSel + 1];     // K row index of every selected token, then the current one
-  int32_t sel_pos[kFusedMaxSel + 1];  // of every selected token: first slot of its group << 16 | offset in its chunk
+  // (+ 64: one spare entry per lane behind each list, where the emission of the final selection puts
+  // the candidates that are not selected instead of branching around them)
+  int32_t rows[kFusedMaxSel + 1 + 64];  // K row index of every selected token, then the current one
+  int32_t sel_pos[kFusedMaxSel + 1 + 64];  // of every selected token: first slot of its group << 16 | offset in its chunk
   FinalSelectShared sel;
   // kFromQkv: the rotated query (scaled for the softmax), the rotated new key and the new value
   alignas(16) float qkv_now[3][kHeadDim];
@@ -439,7 +441,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   };
 
   // ---- final selection among the candidates of this head -------------------------------------------
-  const uint32_t n_take = final_select<kGroups>(
+  const uint32_t n_take = final_select<kGroups, true>(
       crow, n_slots, hist + static_cast<size_t>(bh) * hist_stride * kHistBins, n_chunks, k,
       cand_stride, sh.sel,
       [&](uint32_t pos, uint32_t slot0, uint32_t offset, uint32_t, uint32_t krow)
@@ -451,7 +453,8 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
           },
       [&]() __attribute__((always_inline)) {
         if (kFromQkv) make_q_and_key();
-      });
+      },
+      kFusedMaxSel + 1u);
   int32_t* sdst = sel_out ? sel_out + static_cast<size_t>(bh) * k : nullptr;
   if (!kFromQkv && tid == 0) sh.rows[n_take] = cur_row;  // the current token closes the list
   __syncthreads();
