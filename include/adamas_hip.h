@@ -25,7 +25,8 @@
  * multiple of num_kv_heads; equal in the reference, which asserts it,
  * kernels/include/decode/decode_handler.cuh:83).  Query head h uses key/value head
  * h / (num_heads / num_kv_heads): its distances are taken against that head's codes, its selection is
- * its own, its attention reads that head's rows.
+ * its own, its attention reads that head's rows.  The estimator and the decode step want
+ * num_heads * (num_heads / num_kv_heads) < 65536 (ADAMAS_E_UNSUPPORTED otherwise).
  */
 #ifndef ADAMAS_HIP_H_
 #define ADAMAS_HIP_H_
