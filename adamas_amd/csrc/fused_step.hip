@@ -338,8 +338,18 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
                             });
 }
 
+// Up to 128 rows (one round of loads) the attention of launch 2 runs on the first four waves only (16
+// groups of 16 lanes, 8 rows in flight per group instead of 32 groups with 4 each).  The other four
+// waves leave once the row list is closed: the kernel is bound by instruction issue, and the folding
+// and merging of the group states is paid per wave, so half the waves with twice the rows each cost
+// less (budget 128: 0.05 - 0.2 us).  With a second round of rows all eight waves are faster (budget
+// 256: 0.35 us).
+constexpr int kAttendWaves = 4;
+constexpr int kAttendGroups = 4 * kAttendWaves;
+
 struct SelectAttendShared {
   MergeShared<32> merge;
+  MergeShared<kAttendGroups> merge_few;
   // (+ 64: one spare entry per lane behind each list, where the emission of the final selection puts
   // the candidates that are not selected instead of branching around them)
   int32_t rows[kFusedMaxSel + 1 + 64];  // K row index of every selected token, then the current one
@@ -497,17 +507,20 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   }
 
   // ---- attention over the selected tokens and the current one ------------------------------------
+  const uint32_t n_rows = kFromQkv ? n_take : n_take + 1u;
+  const bool few = n_rows <= kAttendGroups * 8u;  // uniform
+  if (few && wave >= kAttendWaves) return;  // (the barriers below count the waves that are still here)
   HeadKV kv;
   kv.kv_data = kv_data;
   kv.table = nullptr;  // rows are K row indices already
   set_kv_layout_static<kHnd>(kv, kv_head_now, c16, num_kv_heads, page_size);
   kv.seq_len = seq_len;
   SoftmaxState st;
-  attend_rows<32, 4, true, kBf16, true>(kv, qf, g, 0u, kFromQkv ? n_take : n_take + 1u,
-                           [&](uint32_t r) __attribute__((always_inline)) -> int32_t {
-                             return sh.rows[r];
-                           },
-                           st);
+  auto row_of = [&](uint32_t r) __attribute__((always_inline)) -> int32_t { return sh.rows[r]; };
+  if (few)
+    attend_rows<kAttendGroups, 8, true, kBf16, true>(kv, qf, g, 0u, n_rows, row_of, st);
+  else
+    attend_rows<32, 4, true, kBf16, true>(kv, qf, g, 0u, n_rows, row_of, st);
   if (kFromQkv) {
     // the current token, from registers: one more row for group 0
     float d = 0.f;
@@ -524,7 +537,10 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     st.m = m_new;
   }
   float M, L, O;
-  merge_groups<32>(st, g, c16, tid, sh.merge, M, L, O);
+  if (few)
+    merge_groups<kAttendGroups>(st, g, c16, tid, sh.merge_few, M, L, O);
+  else
+    merge_groups<32>(st, g, c16, tid, sh.merge, M, L, O);
   if (tid < kHeadDim) store_elem<kBf16>(out + static_cast<size_t>(bh) * kHeadDim + tid, O / L);
 }
 
