@@ -12,9 +12,10 @@ namespace adamas {
 
 constexpr float kNegBig = -1.0e30f;
 
-// 2^x as the bare hardware instruction.  The library routine exp2f() wraps it in five more instructions that only matter
-// for results below 2^-126, which are weights of zero here; for every other argument the bits are
-// the same.  The attention kernels are bound by instruction issue, and a softmax has many of these.
+// 2^x as the bare hardware instruction.  The library routine exp2f() wraps it in five more
+// instructions that only matter for results below 2^-126, which are weights of zero here; for every
+// other argument the bits are the same.  The attention kernels are bound by instruction issue, and a
+// softmax has many of these.
 __device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <bool kBf16 = false>

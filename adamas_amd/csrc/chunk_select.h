@@ -112,11 +112,12 @@ __device__ __forceinline__ void raw_class_masks(const uint32_t (&keys)[kItems], 
 }
 
 // One wave: the k smallest of its 64 x kItems keys (lane l holds items kItems*l .. kItems*l + kItems-1,
-// any value above 511, e.g. kInvalidKey, = no item; n_valid = number of items).  dst: the chunk's candidate list (cand_stride
-// slots, unused ones are filled with kEmptyCand64); hrow: this lane's 8 bytes of the chunk's
-// histogram row; hist_lds: kChunkHistWords words of LDS owned by this wave, 16-byte aligned; payload(item, i) -> 32
-// bits stored with the candidate (evaluated for selected items only; i = item - kItems * lane is a
-// constant at every call, so a caller can keep its payloads in registers).
+// any value above 511, e.g. kInvalidKey, = no item; n_valid = number of items).  dst: the chunk's
+// candidate list (cand_stride slots, unused ones are filled with kEmptyCand64); hrow: this lane's 8
+// bytes of the chunk's histogram row; hist_lds: kChunkHistWords words of LDS owned by this wave,
+// 16-byte aligned; payload(item, i) -> 32 bits stored with the candidate (evaluated for selected
+// items only; i = item - kItems * lane is a constant at every call, so a caller can keep its
+// payloads in registers).
 // The threshold is read off a histogram instead of being searched for: every lane counts its keys
 // into 512 counters in LDS, a prefix sum over the bins (8 bins per lane, DPP scan
 // across the lanes) finds the bin that holds the k-th smallest key, and the histogram of the
