@@ -50,10 +50,10 @@ _SIGNATURES = {
     "adamas_step_candidates": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32,
                                         c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32,
                                         c_uint32, c_uint32, c_void_p]),
-    "adamas_step_attend": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32,
-                                    c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_uint32,
-                                    c_uint32, c_uint32, c_uint32, c_float, c_uint32, c_uint32,
-                                    c_void_p]),
+    "adamas_step_attend": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    c_uint32, c_void_p, c_void_p, c_void_p, c_size_t, c_uint32,
+                                    c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_uint32,
+                                    c_uint32, c_void_p]),
     "adamas_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
                                c_float, c_void_p]),
     "adamas_rope_split": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_void_p,

@@ -195,6 +195,95 @@ __device__ __forceinline__ void chunk_select_emit(const uint32_t (&keys)[kItems]
   for (uint32_t i = n_take + lane; i < cand_stride; i += kWave) dst[i] = kEmptyCand64;
 }
 
+// Threshold of the k smallest keys from a 512-bin histogram in LDS (one 32-bit counter per key
+// value, 16-byte aligned), computed by one wave; every lane returns the same plan.  Lane l reads
+// bins 8l .. 8l+7 (two 128-bit reads), a DPP prefix sum over the lanes finds the bin that holds the
+// k-th smallest key.  Any number of waves may call this on the same histogram side by side: they
+// only read.
+struct WavePlan {
+  uint32_t thr;      // threshold key (kHistBins when there are at most k keys: all of them are taken)
+  uint32_t n_below;  // keys below the threshold
+  uint32_t quota;    // keys equal to the threshold to take, lowest index first
+  uint32_t n_take;   // k, or the number of keys if that is smaller
+};
+
+__device__ __forceinline__ WavePlan wave_plan_from_hist(const uint32_t* hist_lds, uint32_t k) {
+  const int lane = lane_id();
+  const uint4 hv0 = *reinterpret_cast<const uint4*>(&hist_lds[8 * lane]);
+  const uint4 hv1 = *reinterpret_cast<const uint4*>(&hist_lds[8 * lane + 4]);
+  const uint32_t c[8] = {hv0.x, hv0.y, hv0.z, hv0.w, hv1.x, hv1.y, hv1.z, hv1.w};
+  uint32_t lane_sum = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) lane_sum += c[j];
+  const uint32_t incl = wave_inclusive_scan_dpp(lane_sum);
+  const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), 63));
+  WavePlan p;
+  if (total <= k) {
+    p.thr = static_cast<uint32_t>(kHistBins);
+    p.n_below = total;
+    p.quota = 0;
+    p.n_take = total;
+    return p;
+  }
+  // exactly one bin holds the k-th smallest key; its lane finds it among its 8 bins
+  uint32_t run = incl - lane_sum, t_l = 0, nb_l = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const bool here = run < k && run + c[j] >= k;
+    t_l = here ? 8u * static_cast<uint32_t>(lane) + j : t_l;
+    nb_l = here ? run : nb_l;
+    run += c[j];
+  }
+  const uint64_t cross = __ballot(incl - lane_sum < k && incl >= k);
+  const int src = __builtin_amdgcn_readfirstlane(__ffsll(static_cast<long long>(cross)) - 1);
+  p.thr = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(t_l), src));
+  p.n_below = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(nb_l), src));
+  p.quota = k - p.n_below;
+  p.n_take = k;
+  return p;
+}
+
+// One wave: the kc smallest of its 64 x kItems keys (lane l holds items kItems*l .. kItems*l +
+// kItems-1 in index order; any value above 511 = no item), ties to the lowest index, written to the
+// chunk's candidate list dst[kc] as (key << 48) | (item index << 32) | payload, first the keys below
+// the chunk's threshold, then the tied ones, each class in ascending index order; unused slots are
+// filled with kEmptyCand64.  A list is a prefix of the chunk in (key, index) order: when its last
+// entry is not among the keys a caller finally selects, no key of the chunk outside the list can be.
+// hist_lds: kChunkHistWords words of LDS owned by this wave, 16-byte aligned.  payload(item, i) ->
+// 32 bits stored with the candidate, evaluated for listed items only.
+// kSkipInvalid: items that are no keys are left out of the counting by a branch (worth it where many
+// lanes hold none: they would all add to one spare word); otherwise they count into a spare word
+// without a branch.
+template <int kItems, bool kSkipInvalid, typename Payload>
+__device__ __forceinline__ void chunk_select_capped(const uint32_t (&keys)[kItems], uint32_t kc,
+                                                    uint64_t* dst, uint32_t* hist_lds,
+                                                    Payload&& payload) {
+  const int lane = lane_id();
+  *reinterpret_cast<uint4*>(&hist_lds[8 * lane]) = make_uint4(0u, 0u, 0u, 0u);
+  *reinterpret_cast<uint4*>(&hist_lds[8 * lane + 4]) = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+  for (int i = 0; i < kItems; ++i) {
+    if (kSkipInvalid) {
+      if (keys[i] < static_cast<uint32_t>(kHistBins)) atomicAdd(&hist_lds[keys[i]], 1u);
+    } else {
+      atomicAdd(&hist_lds[min(keys[i], static_cast<uint32_t>(kHistBins))], 1u);
+    }
+  }
+  // the LDS operations of one wave are carried out in order: the counts are complete here
+  const WavePlan p = wave_plan_from_hist(hist_lds, kc);
+  uint32_t below[kItems / 4], equal[kItems / 4];
+  raw_class_masks<kItems>(keys, p.thr, below, equal);
+  uint32_t total;
+  const uint32_t excl = lane_scan<kItems / 4>(below, equal, total);
+  lane_emit<kItems / 4>(below, equal, p.n_below, p.quota, excl & 0xffffu, excl >> 16,
+                        [&](uint32_t pos, int i) __attribute__((always_inline)) {
+                          const uint32_t tok = static_cast<uint32_t>(lane) * kItems + i;
+                          dst[pos] =
+                              (static_cast<uint64_t>((keys[i] << 16) | tok) << 32) | payload(tok, i);
+                        });
+  for (uint32_t i = p.n_take + lane; i < kc; i += kWave) dst[i] = kEmptyCand64;
+}
+
 struct FinalSelectShared {
   uint16_t hpart[kFinalThreads / 32][kHistBins];  // partial histogram sums (16 KB)
   alignas(16) uint32_t wtot[kFinalWaves];         // per-wave totals of the histogram scan

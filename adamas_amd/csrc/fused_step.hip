@@ -1,23 +1,30 @@
 // The whole sparse decode step in two launches (gfx950):
 //
-//   estimate_select_kernel  grid (token chunks, head groups of 8, batch), 512 threads.
-//       A chunk is 512, 1024 or 2048 tokens (the smallest size whose candidate lists fit the second
-//       launch).  Per pass of 512 tokens the workgroup streams the 2-bit codes of 512 tokens x 8 heads
-//       (256 contiguous bytes per token, one 128-bit load per lane, 16 loads in flight per wave; the
-//       loads of the next pass are issued before the distances of the current one are computed),
-//       computes the integer L1 distances to the query code and keeps them in LDS only.  Then one
-//       wave per head selects the (budget-1) nearest tokens of the chunk, exactly, ties to the lowest
-//       index, and writes them as candidates (distance, token offset, K row index) together with a
-//       512-bin byte histogram of their distances.  The distance matrix never reaches HBM.
+//   estimate_select_kernel  grid (token chunks, head groups of 8 or 4, batch), one wave per head.
+//       A sequence is cut into chunks whose lengths differ by at most 16 tokens (StepPlan in
+//       workspace.h: 64 chunks x 4 head groups = one workgroup per CU for a single sequence of 32
+//       heads), so the cost of the launch grows smoothly with the sequence.  Per pass of 512 tokens
+//       the workgroup streams the 2-bit codes of 512 tokens x 8 heads (256 contiguous bytes per
+//       token, one 128-bit load per lane, 16 loads in flight per wave; the loads of the next pass are
+//       issued before the distances of the current one are computed; 16-token units go to the waves
+//       round robin, and in the last pass a wave skips the units its chunk does not have), computes
+//       the integer L1 distances to the query code and keeps them in LDS only.  Then one wave per
+//       head selects the kc nearest tokens of the chunk, exactly, ties to the lowest index, and
+//       writes them as candidates (distance, token offset, K row index).  kc is the budget where the
+//       lists of all chunks fit 1024 slots per head and 16 otherwise.  The distance matrix never
+//       reaches HBM.
 //   select_attend_kernel    grid (heads, batch), 512 threads.
-//       Sums the chunk histograms of its head: the prefix sum gives the global threshold and the tie
-//       quota without any search (the nearest tokens of a sequence are always among the per-chunk
-//       winners).  Candidate lists keep the (below threshold, tied) x ascending-index order and chunks
-//       are concatenated in index order, so "ties to the lowest index" carries over: the selected
-//       candidates are emitted in that order (ranks from DPP prefix scans, no atomics) into an LDS row
-//       list, and the attention runs over them plus the current token: 32 groups of 16 lanes, fp32
-//       online softmax.  Candidates carry their K row index, so no page-table access sits between the
-//       selection and the K/V gather.
+//       Two candidate slots per thread.  A 512-bin histogram of the candidates' distances in LDS
+//       gives the threshold and the tie quota without any search; lists keep the (below threshold,
+//       tied) x ascending-index order and chunks are concatenated in index order, so "ties to the
+//       lowest index" carries over: ranks come from DPP prefix scans, no atomic decides a position.
+//       A list of kc entries is a prefix of its chunk in (distance, index) order: if its last entry
+//       is not selected, nothing the chunk left out can be.  If it is (a chunk that holds more than
+//       kc of the selection: clustered neighbours, or long runs of equal distances), the workgroup
+//       scores that chunk again from its codes and selects among all of its tokens: the result is
+//       exact for any input.  The attention then runs over the selected rows plus the current
+//       token: groups of 16 lanes, fp32 online softmax.  Candidates carry their K row index, so no
+//       page-table access sits between the selection and the K/V gather.
 #include "attend.h"
 #include "codes.h"
 #include "hadamard.h"
@@ -62,6 +69,20 @@ struct QkvSource {
   uint32_t code_flags = 0;
 };
 
+// The chunks of the step (StepPlan): chunk c starts at 16-token unit c*units_q + min(c, units_r) and
+// has units_q + (c < units_r) units; kc candidate slots per (head, chunk).
+struct StepGeom {
+  uint32_t units_q, units_r;
+  uint32_t kc, kc_log2;
+};
+
+__device__ __forceinline__ uint32_t chunk_first_unit(const StepGeom& g, uint32_t c) {
+  return c * g.units_q + min(c, g.units_r);
+}
+__device__ __forceinline__ uint32_t chunk_units(const StepGeom& g, uint32_t c) {
+  return g.units_q + (c < g.units_r ? 1u : 0u);
+}
+
 // Rotary embedding of a row of 128 fp16 held by a wave (lane l = channels 2l and 2l+1) at position
 // pos, in two parts so that a kernel can put other loads between the loads and their first use.
 struct WaveRopeLoads {
@@ -90,30 +111,39 @@ __device__ __forceinline__ void wave_rope_apply(const WaveRopeLoads& r, int lane
   x1 = round_elem<false>(rope_channel(q1, p1, r.cs.y, r.sn.y, upper));
 }
 
-// kHist (budgets beyond the candidate lists): instead of selecting, every wave writes the distances
-// of its head (dist_out [sequence*heads][dist_stride] u16) and a 512-bin histogram of them (16-bit
-// counts, hist_out [sequence*heads][chunks][512]); threshold and positions are then read off the
-// histograms by the integer top-k (topk.hip).  The first head group also writes the K row index of
-// every token (rowmap_out [sequence][dist_stride]), so that the selection can hand row indices to the
-// attention, which then reads no page table.
+// kPartial: chunks may be shorter than kPasses * 512 tokens by whole 16-token units (balanced chunks
+// of a sequence whose length is no multiple of the chunk count): the units of the last pass are
+// tested one by one (uniform over the wave).  Without it every chunk has exactly kPasses * 512 tokens
+// and only the end of the sequence is masked.
+// kHist (budgets beyond the candidate lists, chunks of 512 tokens): instead of selecting, every wave
+// writes the distances of its head (dist_out [sequence*heads][dist_stride] u16) and a 512-bin
+// histogram of them (16-bit counts, hist_out [sequence*heads][chunks][512]); threshold and positions
+// are then read off the histograms by the integer top-k (topk.hip).  The first head group also
+// writes the K row index of every token (rowmap_out [sequence][dist_stride]), so that the selection
+// can hand row indices to the attention, which then reads no page table.
 // kFromQkv: q_code is not read; wave w makes the code of query head w of the group from the fused
 // projection (rotary embedding, Hadamard transform, buckets) while the code loads are in flight.
-template <int kPage, int kPasses, bool kHist = false, int kHeads = kFusedHeads, bool kFromQkv = false>
+// qcode_out (selection mode) [sequence*heads][16]: the query codes this launch worked with, written by
+// the workgroups of chunk 0 for the second launch, which scores truncated chunks again.
+template <int kPage, int kPasses, bool kPartial, bool kHist = false, int kHeads = kFusedHeads,
+          bool kFromQkv = false>
 __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     const uint16_t* __restrict__ q_code, const unsigned char* __restrict__ code_data,
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
-    const int32_t* __restrict__ seq_lens, uint64_t* __restrict__ cand,
-    unsigned char* __restrict__ hist_out, uint32_t hist_stride, uint32_t k, uint32_t cand_stride,
-    uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_inv16, uint32_t page_size_rt,
-    uint32_t table_stride, uint32_t rows_per_page, uint16_t* __restrict__ dist_out = nullptr,
-    int64_t dist_stride = 0, uint32_t* __restrict__ rowmap_out = nullptr,
-    QkvSource src = QkvSource()) {
-  static_assert(!kHist || kPasses == 1, "the histogram mode works on 512-token chunks");
-  constexpr uint32_t kChunk = kFusedBlock * kPasses;  // tokens per workgroup
+    const int32_t* __restrict__ seq_lens, uint64_t* __restrict__ cand, StepGeom geom,
+    uint16_t* __restrict__ qcode_out, uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_inv16,
+    uint32_t page_size_rt, uint32_t table_stride, uint32_t rows_per_page,
+    unsigned char* __restrict__ hist_out = nullptr, uint32_t hist_stride = 0,
+    uint16_t* __restrict__ dist_out = nullptr, int64_t dist_stride = 0,
+    uint32_t* __restrict__ rowmap_out = nullptr, QkvSource src = QkvSource()) {
+  static_assert(!kHist || (kPasses == 1 && !kPartial), "the histogram mode works on 512-token chunks");
   constexpr int kItems = 8 * kPasses;                 // tokens per lane in the selection phase
   static_assert(kHeads == 8 || kHeads == 4, "a token's codes are read by 2 * kHeads lanes");
   constexpr uint32_t kLoadTokens = 32 / kHeads;       // tokens per load instruction: 4 or 8
-  constexpr uint32_t kWaveTokens = 16 * kLoadTokens;  // tokens per wave and pass: 64 or 128
+  constexpr uint32_t kUnitLoads = kStepUnit / kLoadTokens;  // loads per 16-token unit: 4 or 2
+  constexpr uint32_t kWaveUnits = 16 / kUnitLoads;    // units per wave and pass: 4 or 8
+  constexpr uint32_t kPassUnits = kFusedBlock / kStepUnit;  // 32
+  static_assert(kWaveUnits * kHeads == kPassUnits, "the waves of a workgroup cover a pass");
   __shared__ EstimateSelectShared<kPasses, kHeads> sh;
   const uint32_t page_size = kPage ? static_cast<uint32_t>(kPage) : page_size_rt;
   const uint32_t chunk = blockIdx.x, n_chunks = gridDim.x;
@@ -121,38 +151,48 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
   const uint32_t b = blockIdx.z;
   const int lane = lane_id();
   const int wave = wave_id_uniform();
-  const uint32_t chunk_base = chunk * kChunk;
+  const uint32_t unit0 = chunk_first_unit(geom, chunk);
+  const uint32_t n_units = kPartial ? chunk_units(geom, chunk) : kPassUnits * kPasses;
+  const uint32_t chunk_base = unit0 * kStepUnit;
   uint64_t* dst =
       cand + ((static_cast<size_t>(b) * num_heads + hg * kHeads + wave) * n_chunks + chunk) *
-                 cand_stride;
-  // histogram row of this (head, chunk): 512 byte counters, lane l owns bins 8l .. 8l+7
-  uint2* hrow = reinterpret_cast<uint2*>(
-      hist_out + ((static_cast<size_t>(b) * num_heads + hg * kHeads + wave) * hist_stride + chunk) *
-                     kHistBins) + lane;
+                 geom.kc;
 
   constexpr uint32_t kTokLanes = 2 * kHeads;                        // lanes per token
   const uint32_t sub = static_cast<uint32_t>(lane) / kTokLanes;    // token within a load
   const uint32_t hl = (static_cast<uint32_t>(lane) % kTokLanes) >> 1;  // head within the group
   const uint32_t half = static_cast<uint32_t>(lane) & 1u;        // which 64 channels
 
+  // Unit u (of kWaveUnits) of this wave in pass `pass`, counted from the start of the chunk: the
+  // units of a pass go to the waves round robin, so that a short last pass is spread over all waves.
+  auto unit_of = [&](int pass, uint32_t u) __attribute__((always_inline)) -> uint32_t {
+    return static_cast<uint32_t>(pass) * kPassUnits + u * kHeads + static_cast<uint32_t>(wave);
+  };
+  // whether the chunk has that unit (always true except in the last pass of a kPartial launch)
+  auto has_unit = [&](int pass, uint32_t u) __attribute__((always_inline)) -> bool {
+    return !kPartial || pass + 1 < kPasses || unit_of(pass, u) < n_units;
+  };
+
   // Memory round trips before the first code load: with a fixed table stride the sequence length and
   // the page ids are fetched side by side (two dependent levels: table, codes); with an indptr array
   // the table address itself has to be loaded first (three levels).
-  // page ids per pass: one per 16 tokens / per load
-  constexpr int kPageRegs = kPage == 16 ? static_cast<int>(kWaveTokens / 16) : 16;
+  // page ids per pass: one per unit (kPage == 16: a unit is a page, uniform over the wave) or one per load
+  constexpr int kPageRegs = kPage == 16 ? static_cast<int>(kWaveUnits) : 16;
   uint32_t pages[kPasses][kPageRegs];
   const int32_t* table;
   uint32_t lp_max;
   auto lookup_all = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int pass = 0; pass < kPasses; ++pass) {
-      const uint32_t tok0 =
-          chunk_base + pass * kFusedBlock + static_cast<uint32_t>(wave) * kWaveTokens;
 #pragma unroll
       for (int j = 0; j < kPageRegs; ++j) {
-        // kPage == 16: the loads of 16 adjacent tokens share page j (uniform over the wave)
-        const uint32_t lp =
-            kPage == 16 ? (tok0 >> 4) + j : (tok0 + j * kLoadTokens + sub) / page_size;
+        uint32_t lp;
+        if (kPage == 16) {
+          lp = unit0 + unit_of(pass, j);
+        } else {
+          const uint32_t u = static_cast<uint32_t>(j) / kUnitLoads, i = static_cast<uint32_t>(j) % kUnitLoads;
+          lp = (chunk_base + unit_of(pass, u) * kStepUnit + i * kLoadTokens + sub) / page_size;
+        }
         pages[pass][j] = static_cast<uint32_t>(table[min(lp, lp_max)]);
       }
     }
@@ -168,13 +208,12 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
   uint4* hrow16 = reinterpret_cast<uint4*>(
                       hist_out + ((static_cast<size_t>(b) * num_heads + hg * kHeads + wave) *
                                       hist_stride + chunk) * (2 * kHistBins)) + lane;
-  if (chunk_base >= n) {  // no token of this sequence in the chunk: empty candidate lists
+  if (chunk_base >= n) {  // no token of this sequence in the chunk: an empty candidate list
     if (kHist) {
       *hrow16 = make_uint4(0u, 0u, 0u, 0u);
       return;
     }
-    for (uint32_t i = lane; i < cand_stride; i += kWave) dst[i] = kEmptyCand64;
-    *hrow = make_uint2(0u, 0u);
+    for (uint32_t i = lane; i < geom.kc; i += kWave) dst[i] = kEmptyCand64;
     return;
   }
   if (!table_stride) {
@@ -183,7 +222,7 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     lookup_all();
   }
 
-  // ---- distances: per pass, 64 tokens x 8 heads per wave ----------------------------------------
+  // ---- distances: per pass, 16 loads per lane = 64 (or 128) tokens x kHeads heads per wave --------
   {
     const uint32_t head = hg * kHeads + hl;
     QueryPlanes qp;
@@ -198,6 +237,9 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
       const uint4 qraw = *reinterpret_cast<const uint4*>(
           q_code + (static_cast<size_t>(b) * num_heads + head) * kCodeWords + half * 8u);
       qp = make_query_planes(qraw);
+      if (!kHist && chunk == 0 && sub == 0)
+        *reinterpret_cast<uint4*>(qcode_out + (static_cast<size_t>(b) * num_heads + head) * kCodeWords +
+                                  half * 8u) = qraw;
     }
 
     // grouped-query attention: query head h scores the codes of key head h / group; the lanes of a
@@ -207,40 +249,53 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     const uint32_t row_bytes = num_kv_heads * 32u;
     const unsigned char* lane_base = code_data + kv_head_of(head, kv_inv16) * 32u + half * 16u;
 
-    // issues the 16 loads of pass `pass` (tokens pass*512 + wave*64 .. +63 of the chunk); tokens past
-    // the end of the sequence read some valid slot and are masked when the distances are stored
+    // issues the 16 loads of pass `pass`; tokens past the end of the sequence read some valid slot and
+    // are masked when the distances are stored
     auto issue = [&](int pass, uint4 (&kw)[16]) __attribute__((always_inline)) {
-      const uint32_t tok0 = pass * kFusedBlock + static_cast<uint32_t>(wave) * kWaveTokens;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        uint32_t page, in_page;
-        if (kPage == 16) {
-          constexpr int kLoadsPerPage = 16 / kLoadTokens;  // 4 or 2
-          page = pages[pass][j / kLoadsPerPage];
-          in_page = (j % kLoadsPerPage) * kLoadTokens + sub;
-        } else {
-          const uint32_t t = chunk_base + tok0 + j * kLoadTokens + sub;
-          page = pages[pass][j];
-          in_page = t % page_size;
+      for (uint32_t u = 0; u < kWaveUnits; ++u) {
+        if (!has_unit(pass, u)) continue;
+        const uint32_t tok_u = unit_of(pass, u) * kStepUnit;  // first token of the unit, in the chunk
+#pragma unroll
+        for (uint32_t i = 0; i < kUnitLoads; ++i) {
+          const int j = static_cast<int>(u * kUnitLoads + i);
+          uint32_t page, in_page;
+          if (kPage == 16) {
+            page = pages[pass][u];
+            in_page = i * kLoadTokens + sub;
+          } else {
+            page = pages[pass][j];
+            in_page = (chunk_base + tok_u + i * kLoadTokens + sub) % page_size;
+          }
+          kw[j] = *reinterpret_cast<const uint4*>(
+              lane_base + static_cast<size_t>(page * page_size + in_page) * row_bytes);
+          // (written between the loads on purpose: with the 16 loads of a wave back to back the
+          // launch is 0.1 us slower from HBM, although 0.2 us faster from the Infinity Cache)
+          if ((static_cast<uint32_t>(lane) % kTokLanes) == 0)
+            sh.krow[tok_u + i * kLoadTokens + sub] = page * rows_per_page + in_page;
         }
-        kw[j] = *reinterpret_cast<const uint4*>(
-            lane_base + static_cast<size_t>(page * page_size + in_page) * row_bytes);
-        // (written between the loads on purpose: with the 16 loads of a wave back to back the
-        // launch is 0.1 us slower from HBM, although 0.2 us faster from the Infinity Cache)
-        if ((static_cast<uint32_t>(lane) % kTokLanes) == 0)
-          sh.krow[tok0 + j * kLoadTokens + sub] = page * rows_per_page + in_page;
       }
     };
     auto consume = [&](int pass, const uint4 (&kw)[16]) __attribute__((always_inline)) {
-      const uint32_t tok0 = pass * kFusedBlock + static_cast<uint32_t>(wave) * kWaveTokens;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        uint32_t v = l1_64(kw[2 * i], qp) | (l1_64(kw[2 * i + 1], qp) << 16);
-        v += swap_adjacent(v);  // both lanes of a head now hold the distances of loads 2i, 2i+1
-        // the even lane keeps load 2i, the odd lane load 2i+1
-        const uint32_t tok = tok0 + (2 * i + half) * kLoadTokens + sub;
-        const uint32_t d = half ? (v >> 16) : (v & 0xffffu);
-        sh.dist[hl][tok] = (chunk_base + tok < n) ? static_cast<uint16_t>(d) : 0xffffu;
+      for (uint32_t u = 0; u < kWaveUnits; ++u) {
+        const uint32_t tok_u = unit_of(pass, u) * kStepUnit;
+        if (!has_unit(pass, u)) {  // a unit the chunk does not have: no tokens
+#pragma unroll
+          for (uint32_t i2 = 0; i2 < kUnitLoads / 2; ++i2)
+            sh.dist[hl][tok_u + (2 * i2 + half) * kLoadTokens + sub] = 0xffffu;
+          continue;
+        }
+#pragma unroll
+        for (uint32_t i2 = 0; i2 < kUnitLoads / 2; ++i2) {
+          const int j = static_cast<int>(u * kUnitLoads + 2 * i2);
+          uint32_t v = l1_64(kw[j], qp) | (l1_64(kw[j + 1], qp) << 16);
+          v += swap_adjacent(v);  // both lanes of a head now hold the distances of loads j, j+1
+          // the even lane keeps load j, the odd lane load j+1
+          const uint32_t tok = tok_u + (2 * i2 + half) * kLoadTokens + sub;
+          const uint32_t d = half ? (v >> 16) : (v & 0xffffu);
+          sh.dist[hl][tok] = (chunk_base + tok < n) ? static_cast<uint16_t>(d) : 0xffffu;
+        }
       }
     };
     uint4 buf0[16], buf1[16];
@@ -250,7 +305,12 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
       wave_rope_apply(qload, lane, qx0, qx1);
       transform_row(qx0, qx1, lane, src.scale, (src.code_flags & ADAMAS_F_CODE_FROM_FP32) != 0);
       const uint32_t word = wave_pack_codes(qx0, qx1, lane);
-      if ((lane & 3) == 0) sh.qcode[wave][lane >> 2] = static_cast<uint16_t>(word);
+      if ((lane & 3) == 0) {
+        sh.qcode[wave][lane >> 2] = static_cast<uint16_t>(word);
+        if (chunk == 0)
+          qcode_out[(static_cast<size_t>(b) * num_heads + hg * kHeads + wave) * kCodeWords +
+                    (lane >> 2)] = static_cast<uint16_t>(word);
+      }
       // a barrier that waits for the LDS writes only: __syncthreads() would also wait for the 16
       // code loads of every wave before any of them is used
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -302,7 +362,7 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     return;
   }
 
-  // ---- wave w = head w of the group: the k nearest tokens of the chunk ----------------------------
+  // ---- wave w = head w of the group: the kc nearest tokens of the chunk ---------------------------
   // lane l holds tokens kItems*l .. kItems*l + kItems-1 (item order = token order)
   uint32_t keys[kItems];
 #pragma unroll
@@ -311,31 +371,16 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      // 0xffff (no token) stays as it is: above every threshold, and counted into the spare word
+      // 0xffff (no token) stays as it is: above every threshold
       keys[p8 * 8 + 2 * i] = w[i] & 0xffffu;
       keys[p8 * 8 + 2 * i + 1] = w[i] >> 16;
     }
   }
-  // One pass: the K rows of the lane's eight tokens are fetched with the keys (two 128-bit reads), so
-  // that no emitted candidate waits for an LDS round trip of its own.  With more passes the 16 or 32
-  // extra registers cost more than the waits (measured at 131072 tokens), and the rows are read as
-  // they are needed.
-  constexpr bool kRowsAhead = kItems == 8;
-  uint32_t krows[kRowsAhead ? kItems : 1];
-  if (kRowsAhead) {
-#pragma unroll
-    for (int p4 = 0; p4 < kItems / 4; ++p4) {
-      const uint4 v = *reinterpret_cast<const uint4*>(&sh.krow[lane * kItems + p4 * 4]);
-      krows[p4 * 4] = v.x;
-      krows[p4 * 4 + 1] = v.y;
-      krows[p4 * 4 + 2] = v.z;
-      krows[p4 * 4 + 3] = v.w;
-    }
-  }
-  chunk_select_emit<kItems>(keys, min(kChunk, n - chunk_base), k, cand_stride, dst, hrow,
-                            sh.hist[wave], [&](uint32_t tok, int i) __attribute__((always_inline)) {
-                              return kRowsAhead ? krows[kRowsAhead ? i : 0] : sh.krow[tok];
-                            });
+  // the K row of a listed token is read when it is written out (a handful per wave)
+  chunk_select_capped<kItems, kPartial>(keys, geom.kc, dst, sh.hist[wave],
+                                        [&](uint32_t tok, int) __attribute__((always_inline)) {
+                                          return sh.krow[tok];
+                                        });
 }
 
 // Up to 128 rows (one round of loads) the attention of launch 2 runs on the first four waves only (16
@@ -350,34 +395,44 @@ constexpr int kAttendGroups = 4 * kAttendWaves;
 struct SelectAttendShared {
   MergeShared<32> merge;
   MergeShared<kAttendGroups> merge_few;
-  // (+ 64: one spare entry per lane behind each list, where the emission of the final selection puts
-  // the candidates that are not selected instead of branching around them)
-  int32_t rows[kFusedMaxSel + 1 + 64];  // K row index of every selected token, then the current one
-  int32_t sel_pos[kFusedMaxSel + 1 + 64];  // of every selected token: first slot of its group << 16 | offset in its chunk
-  FinalSelectShared sel;
+  int32_t rows[kFusedMaxSel + 1];     // K row index of every selected token, then the current one
+  int32_t sel_pos[kFusedMaxSel + 1];  // position of every selected token
+  alignas(16) uint32_t hist[kHistBins];  // candidates per distance value
+  alignas(16) uint32_t wclass[kAttWaves];  // per-wave class totals of the rank scan: below | tied << 16
+  // chunks whose list is exhausted by the selection and that hold more tokens (scored again):
+  uint32_t flag[kStepMaxChunks];
+  uint32_t any_flag;
+  uint32_t fb[kStepMaxChunks], ft[kStepMaxChunks];  // their tokens below / equal to the threshold
+  uint32_t tbase[kStepMaxChunks];                   // tied list entries of all chunks before them
   // kFromQkv: the rotated query (scaled for the softmax), the rotated new key and the new value
   alignas(16) float qkv_now[3][kHeadDim];
 };
 
-// kGroups: groups of 8 candidate slots per thread (4096 slots per head and group, up to 4 groups)
+// Two candidate slots per thread: slots 2*tid and 2*tid + 1 of the head's n_chunks * kc slots (at
+// most kStepMaxSlots; both belong to one chunk since kc is even).
+// q_code [sequence*heads][16], code_data: the query codes and the code cache the first launch worked
+// with, read only when a chunk has to be scored again; dist_scratch [sequence*heads][dist_stride]
+// u16 then holds that chunk's distances (rows are private to a workgroup).
 // kFromQkv (fp16, NHD pages): q is not read; the kernel takes the fused projection of the decoder,
 // applies the rotary embedding to the query and to the new key itself, appends the new key, its code
 // and the new value (the workgroup of the first query head of a key/value head), and attends the
 // current token from registers instead of reading it back: the decode append needs no launch of its
 // own.
-template <int kGroups, bool kBf16, bool kHnd, bool kFromQkv = false>
+template <bool kBf16, bool kHnd, bool kFromQkv = false>
 __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     const __half* __restrict__ q, const __half* __restrict__ kv_data,
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
-    const int32_t* __restrict__ seq_lens, const uint64_t* __restrict__ cand,
-    const unsigned char* __restrict__ hist, uint32_t hist_stride, uint32_t n_chunks,
-    uint32_t chunk_tokens, uint32_t k, uint32_t cand_stride, __half* __restrict__ out,
-    int32_t* __restrict__ sel_out, uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_group,
-    uint32_t kv_inv16, uint32_t page_size, float scale_log2, uint32_t table_stride,
-    QkvSource src = QkvSource(),
-    __half* kv_append = nullptr, uint16_t* code_data = nullptr) {
+    const int32_t* __restrict__ seq_lens, const uint64_t* __restrict__ cand, StepGeom geom,
+    uint32_t n_chunks, uint32_t k, __half* __restrict__ out, int32_t* __restrict__ sel_out,
+    uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_group, uint32_t kv_inv16,
+    uint32_t page_size, float scale_log2, uint32_t table_stride,
+    const uint16_t* __restrict__ q_code, const unsigned char* code_data,
+    uint16_t* __restrict__ dist_scratch, int64_t dist_stride, QkvSource src = QkvSource(),
+    __half* kv_append = nullptr, uint16_t* code_append = nullptr) {
   static_assert(!kFromQkv || (!kBf16 && !kHnd), "the fused projection is fp16 over NHD pages");
-  static_assert(kAttThreads == kFinalThreads, "final_select runs on the whole workgroup");
+  static_assert(kAttThreads == kHistBins, "one thread per distance value");
+  static_assert(kStepMaxSlots == 2 * kAttThreads, "two candidate slots per thread");
+  static_assert(kStepMaxChunks == kWave, "the flags of all chunks fit one ballot");
   __shared__ SelectAttendShared sh;
   const uint32_t head = blockIdx.x;
   const uint32_t b = blockIdx.y;
@@ -385,7 +440,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   const uint32_t tid = threadIdx.x;
   const int lane = lane_id();
   const int wave = wave_id_uniform();
-  const uint32_t n_slots = n_chunks * cand_stride;  // <= 1024 * kItems, multiple of 8
+  const uint32_t n_slots = n_chunks << geom.kc_log2;
   const uint64_t* crow = cand + static_cast<size_t>(bh) * n_slots;
 
   // K row of the current token: a chain of three dependent scalar loads, started first so that it
@@ -397,25 +452,35 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
       for (uint32_t i = tid; i < k; i += kAttThreads) sel_out[static_cast<size_t>(bh) * k + i] = -1;
     return;
   }
+  const uint32_t n = static_cast<uint32_t>(seq_len) - 1u;  // past tokens
+  const int32_t* table = page_indices + (table_stride ? static_cast<size_t>(b) * table_stride
+                                                      : static_cast<size_t>(page_indptr[b]));
+  const uint32_t rows_per_page = kHnd ? 2u * page_size * num_kv_heads : 2u * page_size;
   int32_t cur_row;
   uint32_t cur_page, cur_slot;
   {
-    const int32_t* table = page_indices + (table_stride ? static_cast<size_t>(b) * table_stride
-                                                        : static_cast<size_t>(page_indptr[b]));
-    const uint32_t p = static_cast<uint32_t>(seq_len) - 1u;
-    const uint32_t lp = p / page_size;
-    const uint32_t rows_per_page = kHnd ? 2u * page_size * num_kv_heads : 2u * page_size;
+    const uint32_t lp = n / page_size;
     cur_page = static_cast<uint32_t>(table[lp]);
-    cur_slot = p - lp * page_size;
+    cur_slot = n - lp * page_size;
     cur_row = static_cast<int32_t>(cur_page * rows_per_page + cur_slot);
   }
+
+  // ---- the candidates of this head: two slots per thread --------------------------------------------
+  const uint32_t slot0 = 2u * tid;
+  const bool have = slot0 < n_slots;
+  uint4 raw = make_uint4(~0u, ~0u, ~0u, ~0u);  // an unused slot is all ones
+  if (have) raw = *reinterpret_cast<const uint4*>(crow + slot0);  // lists are 64-byte aligned
+  sh.hist[tid] = 0u;
+  if (tid < kStepMaxChunks) sh.flag[tid] = 0u;
+  if (tid == 0) sh.any_flag = 0u;
+
   const uint32_t g = tid >> 4;    // group of 16 lanes (32 groups)
   const uint32_t c16 = tid & 15;  // channels [8*c16, 8*c16 + 8)
   float qf[8];
   float kcur[8], vcur[8];  // kFromQkv: the new key (rotated) and value, channels 8*c16 .. +7
   // kFromQkv: wave 0 takes the query row of the projection, wave 1 the new key row, wave 2 the new
-  // value row (lane l = channels 2l and 2l+1).  The loads are issued here and used inside the
-  // selection, once its own loads are under way; the results go to the other waves through LDS.
+  // value row (lane l = channels 2l and 2l+1).  The loads are issued here and used once the
+  // candidates have been counted; the results go to the other waves through LDS.
   WaveRopeLoads row_now = {};
   const uint32_t kv_head_now = kv_head_of(head, kv_inv16);  // kv_group = num_heads / num_kv_heads
   // the waves that append the new token of this head's key/value head (one workgroup per key/value head)
@@ -427,14 +492,23 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
       const uint32_t sel_row = wave == 0 ? head
                                : wave == 1 ? num_heads + kv_head_now
                                            : num_heads + num_kv_heads + kv_head_now;
-      row_now = wave_rope_load(row + static_cast<size_t>(sel_row) * kHeadDim, src,
-                               static_cast<uint32_t>(seq_len) - 1u, lane);
+      row_now = wave_rope_load(row + static_cast<size_t>(sel_row) * kHeadDim, src, n, lane);
     }
   } else {
     load_query<kBf16>(q + static_cast<size_t>(bh) * kHeadDim, c16, scale_log2, qf);
   }
-  auto make_q_and_key = [&]() __attribute__((always_inline)) {
-    if (wave >= 3) return;
+
+  // a candidate is (distance << 48) | (token offset in its chunk << 32) | K row index
+  uint32_t key[2] = {raw.y >> 16, raw.w >> 16};  // an unused slot reads 0xffff: above every threshold
+  const uint32_t off[2] = {raw.y & 0xffffu, raw.w & 0xffffu};
+  const uint32_t krow[2] = {raw.x, raw.z};
+  const uint32_t chunk_mine = slot0 >> geom.kc_log2;
+  const uint32_t chunk_tok0 = chunk_first_unit(geom, chunk_mine) * kStepUnit;
+  __syncthreads();  // the histogram is cleared
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (key[i] < static_cast<uint32_t>(kHistBins)) atomicAdd(&sh.hist[key[i]], 1u);
+  if (kFromQkv && wave < 3) {
     float x0, x1;
     if (wave == 2) {  // the value row is taken as it is
       unpack2<false>(row_now.raw, x0, x1);
@@ -448,34 +522,176 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
       transform_row(x0, x1, lane, src.scale, (src.code_flags & ADAMAS_F_CODE_FROM_FP32) != 0);
       kcode_word = wave_pack_codes(x0, x1, lane);
     }
-  };
+  }
+  __syncthreads();  // the histogram is complete
 
-  // ---- final selection among the candidates of this head -------------------------------------------
-  const uint32_t n_take = final_select<kGroups, true>(
-      crow, n_slots, hist + static_cast<size_t>(bh) * hist_stride * kHistBins, n_chunks, k,
-      cand_stride, sh.sel,
-      [&](uint32_t pos, uint32_t slot0, uint32_t offset, uint32_t, uint32_t krow)
-          __attribute__((always_inline)) {
-            sh.rows[pos] = static_cast<int32_t>(krow);
-            // slot (< 2^15) and offset in the chunk (< 2^16): turned into a position only when
-            // the caller asked for the selection
-            sh.sel_pos[pos] = static_cast<int32_t>((slot0 << 16) | offset);
-          },
-      [&]() __attribute__((always_inline)) {
-        if (kFromQkv) make_q_and_key();
-      },
-      kFusedMaxSel + 1u);
-  int32_t* sdst = sel_out ? sel_out + static_cast<size_t>(bh) * k : nullptr;
-  if (!kFromQkv && tid == 0) sh.rows[n_take] = cur_row;  // the current token closes the list
-  __syncthreads();
-  // the selection goes out once the row list is complete (every wave has emitted its part)
-  if (sdst)
-    for (uint32_t i = tid; i < k; i += kAttThreads) {
-      const uint32_t v = static_cast<uint32_t>(sh.sel_pos[i]);
-      sdst[i] = i < n_take
-                    ? static_cast<int32_t>((v >> 16) / cand_stride * chunk_tokens + (v & 0xffffu))
-                    : -1;
+  // ---- selection among the listed candidates ----------------------------------------------------------
+  // every wave reads the threshold off the histogram for itself (no exchange)
+  WavePlan plan = wave_plan_from_hist(sh.hist, k);
+  // Ranks of this thread's two slots: `rb` listed candidates below the threshold and `re` tied ones
+  // come before them in slot order (wave prefix scan + the totals of the earlier waves).
+  uint32_t rb, re, list_below;
+  auto rank_slots = [&]() __attribute__((always_inline)) {
+    const uint32_t mine = (key[0] < plan.thr ? 1u : 0u) + (key[1] < plan.thr ? 1u : 0u) +
+                          (((key[0] == plan.thr ? 1u : 0u) + (key[1] == plan.thr ? 1u : 0u)) << 16);
+    const uint32_t incl = wave_inclusive_scan_dpp(mine);
+    if (lane == kWave - 1) sh.wclass[wave] = incl;
+    __syncthreads();
+    static_assert(kAttWaves == 8, "two 128-bit reads cover the wave totals");
+    const uint4 lo = *reinterpret_cast<const uint4*>(&sh.wclass[0]);
+    const uint4 hi = *reinterpret_cast<const uint4*>(&sh.wclass[4]);
+    const uint32_t t[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    uint32_t before = 0, all = 0;  // the 16-bit fields cannot carry: at most 1024 slots
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      before += w < wave ? t[w] : 0u;
+      all += t[w];
     }
+    const uint32_t excl = before + incl - mine;
+    rb = excl & 0xffffu;
+    re = excl >> 16;
+    list_below = all & 0xffffu;
+  };
+  const bool want_pos = sel_out != nullptr;
+  // writes the selected ones of this thread's slots into the row list; `tie_shift` tied tokens of
+  // re-scored chunks come before this thread's chunk.  Returns whether the second slot was selected.
+  auto emit_slots = [&](uint32_t tie_shift) __attribute__((always_inline)) -> bool {
+    uint32_t pb = rb, pe = re + tie_shift;
+    bool last_selected = false;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const bool is_b = key[i] < plan.thr, is_e = key[i] == plan.thr;
+      const bool take = is_b || (is_e && pe < plan.quota);
+      if (take) {
+        const uint32_t pos = is_b ? pb : plan.n_below + pe;
+        sh.rows[pos] = static_cast<int32_t>(krow[i]);
+        if (want_pos) sh.sel_pos[pos] = static_cast<int32_t>(chunk_tok0 + off[i]);
+      }
+      pb += is_b ? 1u : 0u;
+      pe += is_e ? 1u : 0u;
+      last_selected = take;
+    }
+    return last_selected;
+  };
+  rank_slots();
+  {
+    const bool last_selected = emit_slots(0u);
+    // The list of a chunk is a prefix of the chunk in (distance, index) order.  If its last entry is
+    // selected and the chunk holds more tokens than the list, tokens outside the list may belong to
+    // the selection too: the chunk is scored again below.
+    if (last_selected && ((slot0 + 1u) & (geom.kc - 1u)) == geom.kc - 1u) {
+      const uint32_t chunk_len = min(chunk_units(geom, chunk_mine) * kStepUnit, n - chunk_tok0);
+      if (chunk_len > geom.kc) {
+        sh.flag[chunk_mine] = 1u;
+        sh.any_flag = 1u;
+      }
+    }
+  }
+  if (!kFromQkv && tid == 0) sh.rows[plan.n_take] = cur_row;  // the current token closes the list
+  __syncthreads();  // the row list is complete, or some chunk is flagged
+
+  if (sh.any_flag) {
+    // ---- some lists were too short: score those chunks again and select among all their tokens -------
+    // (at most (budget-1) / kc chunks: every one of them has kc selected entries)
+    const uint64_t fmask = __ballot(sh.flag[lane] != 0u);  // the same in every wave
+    const bool mine_flagged = have && ((fmask >> chunk_mine) & 1ull) != 0;
+    if (mine_flagged) {  // the listed entries of such a chunk leave the count: its tokens come back below
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (key[i] < static_cast<uint32_t>(kHistBins)) atomicSub(&sh.hist[key[i]], 1u);
+        key[i] = 0xffffu;
+      }
+    }
+    const uint16_t* qc = q_code + static_cast<size_t>(bh) * kCodeWords;
+    const QueryPlanes qp_lo = make_query_planes(*reinterpret_cast<const uint4*>(qc));
+    const QueryPlanes qp_hi = make_query_planes(*reinterpret_cast<const uint4*>(qc + 8));
+    uint16_t* drow = dist_scratch + static_cast<size_t>(bh) * dist_stride;
+    const uint32_t code_row_bytes = num_kv_heads * 32u;
+    for (uint64_t m = fmask; m; m &= m - 1) {
+      const uint32_t c = static_cast<uint32_t>(__ffsll(static_cast<long long>(m)) - 1);
+      const uint32_t t0 = chunk_first_unit(geom, c) * kStepUnit;
+      const uint32_t len = min(chunk_units(geom, c) * kStepUnit, n - t0);
+      for (uint32_t t = tid; t < len; t += kAttThreads) {
+        const uint32_t pos = t0 + t;
+        const uint32_t lp = pos / page_size;
+        const uint32_t tslot = static_cast<uint32_t>(table[lp]) * page_size + (pos - lp * page_size);
+        const unsigned char* cp =
+            code_data + static_cast<size_t>(tslot) * code_row_bytes + kv_head_now * 32u;
+        const uint32_t d = l1_64(*reinterpret_cast<const uint4*>(cp), qp_lo) +
+                           l1_64(*reinterpret_cast<const uint4*>(cp + 16), qp_hi);
+        drow[pos] = static_cast<uint16_t>(d);
+        atomicAdd(&sh.hist[d], 1u);
+      }
+    }
+    __syncthreads();  // counts complete; the distances written above are visible to the workgroup
+    plan = wave_plan_from_hist(sh.hist, k);
+    // wave w counts the tokens below / equal to the new threshold in the flagged chunks w, w+8, ...
+    {
+      uint32_t f = 0;
+      for (uint64_t m = fmask; m; m &= m - 1, ++f) {
+        if ((f & (kAttWaves - 1)) != static_cast<uint32_t>(wave)) continue;
+        const uint32_t c = static_cast<uint32_t>(__ffsll(static_cast<long long>(m)) - 1);
+        const uint32_t t0 = chunk_first_unit(geom, c) * kStepUnit;
+        const uint32_t len = min(chunk_units(geom, c) * kStepUnit, n - t0);
+        uint32_t cb = 0, ce = 0;
+        for (uint32_t t = 0; t < len; t += kWave) {
+          const uint32_t d = t + lane < len ? static_cast<uint32_t>(drow[t0 + t + lane]) : 0xffffu;
+          cb += __popcll(__ballot(d < plan.thr));
+          ce += __popcll(__ballot(d == plan.thr));
+        }
+        if (lane == 0) {
+          sh.fb[c] = cb;
+          sh.ft[c] = ce;
+        }
+      }
+    }
+    rank_slots();  // (its barrier also publishes fb and ft)
+    // listed ties of all chunks in front of a flagged chunk: what its first slot's thread counted
+    if (mine_flagged && (slot0 & (geom.kc - 1u)) == 0u) sh.tbase[chunk_mine] = re;
+    uint32_t tie_shift = 0;  // tied tokens of flagged chunks in front of this thread's chunk
+    for (uint64_t m = have ? fmask & ((1ull << chunk_mine) - 1ull) : 0ull; m; m &= m - 1)
+      tie_shift += sh.ft[__ffsll(static_cast<long long>(m)) - 1];
+    __syncthreads();
+    emit_slots(tie_shift);
+    // the flagged chunks, walked in token order by their waves: tokens below the threshold go behind
+    // the listed ones, tied tokens take the rank their index gives them among all ties
+    {
+      uint32_t f = 0, bb = list_below, tb = 0;
+      for (uint64_t m = fmask; m; m &= m - 1, ++f) {
+        const uint32_t c = static_cast<uint32_t>(__ffsll(static_cast<long long>(m)) - 1);
+        if ((f & (kAttWaves - 1)) == static_cast<uint32_t>(wave)) {
+          const uint32_t t0 = chunk_first_unit(geom, c) * kStepUnit;
+          const uint32_t len = min(chunk_units(geom, c) * kStepUnit, n - t0);
+          uint32_t pb = bb, pe = sh.tbase[c] + tb;
+          for (uint32_t t = 0; t < len; t += kWave) {
+            const uint32_t pos = t0 + t + lane;
+            const uint32_t d = t + lane < len ? static_cast<uint32_t>(drow[pos]) : 0xffffu;
+            const uint64_t mb = __ballot(d < plan.thr), me = __ballot(d == plan.thr);
+            const uint32_t r_e = pe + lanes_below(me);
+            const bool is_b = d < plan.thr;
+            if (is_b || (d == plan.thr && r_e < plan.quota)) {
+              const uint32_t dst_pos = is_b ? pb + lanes_below(mb) : plan.n_below + r_e;
+              const uint32_t lp = pos / page_size;
+              sh.rows[dst_pos] = static_cast<int32_t>(static_cast<uint32_t>(table[lp]) * rows_per_page +
+                                                      (pos - lp * page_size));
+              if (want_pos) sh.sel_pos[dst_pos] = static_cast<int32_t>(pos);
+            }
+            pb += __popcll(mb);
+            pe += __popcll(me);
+          }
+        }
+        bb += sh.fb[c];
+        tb += sh.ft[c];
+      }
+    }
+    if (!kFromQkv && tid == 0) sh.rows[plan.n_take] = cur_row;
+    __syncthreads();  // the row list is complete
+  }
+  const uint32_t n_take = plan.n_take;
+  if (want_pos) {
+    int32_t* sdst = sel_out + static_cast<size_t>(bh) * k;
+    for (uint32_t i = tid; i < k; i += kAttThreads) sdst[i] = i < n_take ? sh.sel_pos[i] : -1;
+  }
   if (kFromQkv) {
     // the query for every group, the new key and value for the group that attends them
     const float4 a0 = *reinterpret_cast<const float4*>(&sh.qkv_now[0][8 * c16]);
@@ -488,8 +704,8 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
       vcur[j] = sh.qkv_now[2][8 * c16 + j];
     }
     if (appends && (wave == 1 || wave == 2)) {
-      // the new token goes into the caches, likewise after the last barrier: wave 1 writes K
-      // (rotated) and its code, wave 2 writes V
+      // the new token goes into the caches after every read of them: wave 1 writes K (rotated) and
+      // its code, wave 2 writes V
       const size_t tok_stride = static_cast<size_t>(num_kv_heads) * kHeadDim;
       __half* krow_p = kv_append +
                        (static_cast<size_t>(cur_page) * 2 * page_size + cur_slot) * tok_stride +
@@ -497,8 +713,8 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
       if (wave == 1) {
         reinterpret_cast<uint32_t*>(krow_p)[lane] = kpacked;
         if ((lane & 3) == 0)
-          code_data[((static_cast<size_t>(cur_page) * page_size + cur_slot) * num_kv_heads +
-                     kv_head_now) * kCodeWords + (lane >> 2)] = static_cast<uint16_t>(kcode_word);
+          code_append[((static_cast<size_t>(cur_page) * page_size + cur_slot) * num_kv_heads +
+                       kv_head_now) * kCodeWords + (lane >> 2)] = static_cast<uint16_t>(kcode_word);
       } else {
         reinterpret_cast<uint32_t*>(krow_p + static_cast<size_t>(page_size) * tok_stride)[lane] =
             row_now.raw;
@@ -548,9 +764,8 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
 
 using namespace adamas;
 
-// the two-launch path serves budgets up to 256 and sequences whose candidate lists fit the final
-// pass; workspace_layout() decides and sizes the candidate buffers accordingly
-static bool fused_eligible(const WorkspaceLayout& w) { return w.fused_ok != 0; }
+// the two-launch path serves budgets up to 256 and sequences the plan of workspace.h covers
+static bool fused_eligible(const WorkspaceLayout& w) { return w.plan.ok != 0; }
 
 extern "C" int adamas_step_fused_supported(uint32_t batch, uint32_t num_heads,
                                            uint32_t max_seq_len, uint32_t budget) {
@@ -559,44 +774,18 @@ extern "C" int adamas_step_fused_supported(uint32_t batch, uint32_t num_heads,
   return fused_eligible(workspace_layout(batch, num_heads, max_seq_len, budget)) ? 1 : 0;
 }
 
-// CUs of the current device (asked once per device)
-static uint32_t device_cu_count() {
-  static std::atomic<uint32_t> cached[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  uint32_t n = cached[dev].load(std::memory_order_relaxed);
-  if (n == 0) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
-      v = 256;
-    n = static_cast<uint32_t>(v);
-    cached[dev].store(n, std::memory_order_relaxed);
-  }
-  return n;
-}
-
-// Heads per workgroup of the estimator for a launch of `chunks` chunks per head group.  A CU serves
-// the loads of its workgroups in order, so the launch lasts as long as the CU with the most bytes:
-// with n wide workgroups on C CUs that is ceil(n / C) of them, with 2n narrow ones ceil(2n / C) / 2.
-// The narrow workgroup (4 heads, 128 contiguous bytes per token) is taken where that is less -
-// launches that do not fill the chip (4096 tokens: 6.3 -> 5.0 us, 16384: 7.2 -> 6.5) or spill a few
-// workgroups past a full round (32800 tokens: 12.4 -> 11.5 us) -
-// and the wide one (256 bytes per token) otherwise (32768 tokens: 10.2 against 10.3 us, 131072
-// tokens: 32.7 against 34.4).
-static int estimator_heads(uint32_t chunks, uint32_t num_heads, uint32_t batch) {
-  const uint64_t cus = device_cu_count();
-  const uint64_t wide = static_cast<uint64_t>(chunks) * (num_heads / kFusedHeads) * batch;
-  const uint64_t rounds_wide = (wide + cus - 1) / cus;            // in wide workgroups
-  const uint64_t rounds_narrow2 = (2 * wide + cus - 1) / cus;     // in half workgroups
-  // several sequences: their lengths differ (only the device knows by how much), chunks past the end
-  // of a sequence leave at once, and the finer unit balances better (the batch of 16: 90.0 -> 88.0 us)
-  if (batch > 1) return 4;
-  return rounds_narrow2 < 2 * rounds_wide ? 4 : kFusedHeads;
-}
-
 // rows per page of the KV layout the K row indices are meant for
 static uint32_t rows_per_page_of(uint32_t flags, uint32_t page_size, uint32_t num_kv_heads) {
   return make_kv_layout((flags & ADAMAS_F_HND) != 0, page_size, num_kv_heads).rows_per_page;
+}
+
+static StepGeom geom_of(const StepPlan& p) {
+  StepGeom g;
+  g.units_q = p.units_q;
+  g.units_r = p.units_r;
+  g.kc = p.kc;
+  g.kc_log2 = p.kc_log2;
+  return g;
 }
 
 // qsrc != nullptr: the query codes are made in the kernel from the fused projection (q_code unused)
@@ -625,46 +814,56 @@ static int step_candidates_impl(const void* q_code, const void* code_data,
   if (!fused_eligible(w)) return ADAMAS_E_UNSUPPORTED;
   char* ws = static_cast<char*>(workspace);
   uint64_t* cand = reinterpret_cast<uint64_t*>(ws + w.cand_off);
-  unsigned char* hist = reinterpret_cast<unsigned char*>(ws + w.hist_off);
-  const int est_heads = estimator_heads(w.cand_chunks, num_heads, batch);
-  const dim3 grid(w.cand_chunks, num_heads / est_heads, batch);
+  uint16_t* qcode_ws = reinterpret_cast<uint16_t*>(ws + w.qcode_off);
+  const StepPlan& plan = w.plan;
+  const int est_heads = static_cast<int>(plan.heads);
+  const dim3 grid(plan.chunks, num_heads / est_heads, batch);
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define ADAMAS_LAUNCH_ESTSEL_Q(PG, PASSES, HEADS, FROMQKV)                                      \
-  hipLaunchKernelGGL((estimate_select_kernel<PG, PASSES, false, HEADS, FROMQKV>), grid,         \
+#define ADAMAS_LAUNCH_ESTSEL_Q(PG, PASSES, PARTIAL, HEADS, FROMQKV)                             \
+  hipLaunchKernelGGL((estimate_select_kernel<PG, PASSES, PARTIAL, false, HEADS, FROMQKV>), grid, \
                      dim3(HEADS * kWave), 0, s,                                                 \
                      static_cast<const uint16_t*>(q_code),                                    \
                      static_cast<const unsigned char*>(code_data), page_indices, page_indptr, \
-                     seq_lens, cand, hist, w.hist_stride, budget - 1, w.cand_stride,          \
+                     seq_lens, cand, geom_of(plan), qcode_ws,                                 \
                      num_heads, num_kv_heads, group_inv16(num_heads / num_kv_heads),         \
                      page_size, page_table_stride,                                            \
                      rows_per_page_of(flags, page_size, num_kv_heads),                        \
+                     static_cast<unsigned char*>(nullptr), 0u,                                \
                      static_cast<uint16_t*>(nullptr), static_cast<int64_t>(0),                \
                      static_cast<uint32_t*>(nullptr), qsrc ? *qsrc : QkvSource())
-#define ADAMAS_LAUNCH_ESTSEL_H(PG, PASSES, HEADS)        \
-  if (qsrc) {                                            \
-    ADAMAS_LAUNCH_ESTSEL_Q(PG, PASSES, HEADS, true);     \
-  } else {                                               \
-    ADAMAS_LAUNCH_ESTSEL_Q(PG, PASSES, HEADS, false);    \
+#define ADAMAS_LAUNCH_ESTSEL_H(PG, PASSES, PARTIAL, HEADS)        \
+  if (qsrc) {                                                     \
+    ADAMAS_LAUNCH_ESTSEL_Q(PG, PASSES, PARTIAL, HEADS, true);     \
+  } else {                                                        \
+    ADAMAS_LAUNCH_ESTSEL_Q(PG, PASSES, PARTIAL, HEADS, false);    \
   }
-#define ADAMAS_LAUNCH_ESTSEL(PG, PASSES)       \
-  if (est_heads == 4) {                        \
-    ADAMAS_LAUNCH_ESTSEL_H(PG, PASSES, 4)      \
-  } else {                                     \
-    ADAMAS_LAUNCH_ESTSEL_H(PG, PASSES, 8)      \
+#define ADAMAS_LAUNCH_ESTSEL(PG, PASSES, PARTIAL)       \
+  if (est_heads == 4) {                                 \
+    ADAMAS_LAUNCH_ESTSEL_H(PG, PASSES, PARTIAL, 4)      \
+  } else {                                              \
+    ADAMAS_LAUNCH_ESTSEL_H(PG, PASSES, PARTIAL, 8)      \
   }
-#define ADAMAS_LAUNCH_ESTSEL_PAGE(PASSES)   \
-  if (page_size == 16) {                    \
-    ADAMAS_LAUNCH_ESTSEL(16, PASSES)        \
-  } else {                                  \
-    ADAMAS_LAUNCH_ESTSEL(0, PASSES)         \
+#define ADAMAS_LAUNCH_ESTSEL_PAGE(PASSES, PARTIAL)   \
+  if (page_size == 16) {                             \
+    ADAMAS_LAUNCH_ESTSEL(16, PASSES, PARTIAL)        \
+  } else {                                           \
+    ADAMAS_LAUNCH_ESTSEL(0, PASSES, PARTIAL)         \
   }
-  const uint32_t passes = w.chunk_tokens / kFusedBlock;
-  if (passes == 1) {
-    ADAMAS_LAUNCH_ESTSEL_PAGE(1)
-  } else if (passes == 2) {
-    ADAMAS_LAUNCH_ESTSEL_PAGE(2)
+  // chunks of exactly 512, 1024 or 2048 tokens have instances without the per-unit tests
+  if (!plan.partial && plan.passes == 1) {
+    ADAMAS_LAUNCH_ESTSEL_PAGE(1, false)
+  } else if (!plan.partial && plan.passes == 2) {
+    ADAMAS_LAUNCH_ESTSEL_PAGE(2, false)
+  } else if (!plan.partial && plan.passes == 4) {
+    ADAMAS_LAUNCH_ESTSEL_PAGE(4, false)
+  } else if (plan.passes == 1) {
+    return ADAMAS_E_UNSUPPORTED;  // (no plan has a partial single pass: its chunks are 512 tokens)
+  } else if (plan.passes == 2) {
+    ADAMAS_LAUNCH_ESTSEL_PAGE(2, true)
+  } else if (plan.passes == 3) {
+    ADAMAS_LAUNCH_ESTSEL_PAGE(3, true)
   } else {
-    ADAMAS_LAUNCH_ESTSEL_PAGE(4)
+    ADAMAS_LAUNCH_ESTSEL_PAGE(4, true)
   }
 #undef ADAMAS_LAUNCH_ESTSEL_PAGE
 #undef ADAMAS_LAUNCH_ESTSEL
@@ -700,22 +899,23 @@ extern "C" int adamas_step_candidates(const void* q_code, const void* code_data,
 
 // qsrc != nullptr (fp16, NHD): q is made in the kernel from the fused projection, the new token is
 // appended by it (kv_data and code_data are written)
-static int step_attend_impl(const void* q, void* kv_data, const int32_t* page_indices,
+static int step_attend_impl(const void* q, void* kv_data, void* code_data,
+                            const int32_t* page_indices,
                             const int32_t* page_indptr, const int32_t* seq_lens, uint32_t budget,
                             void* out, int32_t* sel_out, void* workspace, size_t workspace_bytes,
                             uint32_t batch, uint32_t num_heads, uint32_t num_kv_heads,
                             uint32_t head_dim, uint32_t page_size, float sm_scale,
                             uint32_t max_seq_len, uint32_t page_table_stride, uint32_t flags,
-                            adamas_stream_t stream, const QkvSource* qsrc, void* code_data) {
+                            adamas_stream_t stream, const QkvSource* qsrc) {
   if (flags & ~(ADAMAS_F_BF16 | ADAMAS_F_HND)) return ADAMAS_E_BADARG;
   if (qsrc) {
-    if (flags != 0 || !code_data) return ADAMAS_E_UNSUPPORTED;
+    if (flags != 0) return ADAMAS_E_UNSUPPORTED;
     q = qsrc->qkv;
   }
   const bool bf16 = (flags & ADAMAS_F_BF16) != 0;
   const bool hnd = (flags & ADAMAS_F_HND) != 0;
-  if (!q || !kv_data || !page_indices || (!page_indptr && !page_table_stride) || !seq_lens ||
-      !out || !workspace ||
+  if (!q || !kv_data || !code_data || !page_indices || (!page_indptr && !page_table_stride) ||
+      !seq_lens || !out || !workspace ||
       budget == 0 || max_seq_len == 0 || batch == 0 || page_size == 0)
     return ADAMAS_E_BADARG;
   if (head_dim != kHeadDim || num_heads == 0 || num_heads % 32 != 0 || batch > 65535)
@@ -724,55 +924,46 @@ static int step_attend_impl(const void* q, void* kv_data, const int32_t* page_in
   // the kernels take head / group from a 16-bit reciprocal (kv_head_of)
   if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(workspace) & 255) return ADAMAS_E_ALIGN;
-  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kv_data)) & 15)
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kv_data) |
+       reinterpret_cast<uintptr_t>(code_data)) & 15)
     return ADAMAS_E_ALIGN;
   const WorkspaceLayout w = workspace_layout(batch, num_heads, max_seq_len, budget);
   if (workspace_bytes < w.total) return ADAMAS_E_WORKSPACE;
   if (!fused_eligible(w)) return ADAMAS_E_UNSUPPORTED;
   char* ws = static_cast<char*>(workspace);
-#define ADAMAS_LAUNCH_SELATT_BF(G, BF, HND, FROMQKV)                                             \
-  hipLaunchKernelGGL((select_attend_kernel<G, BF, HND, FROMQKV>), dim3(num_heads, batch),        \
+  const StepPlan& plan = w.plan;
+#define ADAMAS_LAUNCH_SELATT_BF(BF, HND, FROMQKV)                                                \
+  hipLaunchKernelGGL((select_attend_kernel<BF, HND, FROMQKV>), dim3(num_heads, batch),           \
                      dim3(kAttThreads), 0,                                                       \
                      static_cast<hipStream_t>(stream), static_cast<const __half*>(q),           \
                      static_cast<const __half*>(kv_data), page_indices, page_indptr, seq_lens,  \
-                     reinterpret_cast<const uint64_t*>(ws + w.cand_off),                        \
-                     reinterpret_cast<const unsigned char*>(ws + w.hist_off), w.hist_stride,    \
-                     w.cand_chunks, w.chunk_tokens, budget - 1, w.cand_stride,                  \
-                     static_cast<__half*>(out), sel_out, num_heads, num_kv_heads,               \
-                     num_heads / num_kv_heads, group_inv16(num_heads / num_kv_heads), page_size, \
-                     sm_scale * 1.4426950408889634f, page_table_stride,                          \
-                     qsrc ? *qsrc : QkvSource(), static_cast<__half*>(kv_data),                  \
+                     reinterpret_cast<const uint64_t*>(ws + w.cand_off), geom_of(plan),         \
+                     plan.chunks, budget - 1, static_cast<__half*>(out), sel_out, num_heads,    \
+                     num_kv_heads, num_heads / num_kv_heads,                                    \
+                     group_inv16(num_heads / num_kv_heads), page_size,                          \
+                     sm_scale * 1.4426950408889634f, page_table_stride,                         \
+                     reinterpret_cast<const uint16_t*>(ws + w.qcode_off),                       \
+                     static_cast<const unsigned char*>(code_data),                              \
+                     reinterpret_cast<uint16_t*>(ws + w.dist_off), w.dist_stride,               \
+                     qsrc ? *qsrc : QkvSource(), static_cast<__half*>(kv_data),                 \
                      static_cast<uint16_t*>(code_data))
-#define ADAMAS_LAUNCH_SELATT(G)        \
-  if (qsrc) {                                        \
-    ADAMAS_LAUNCH_SELATT_BF(G, false, false, true);  \
-  } else if (bf16 && hnd) {                          \
-    ADAMAS_LAUNCH_SELATT_BF(G, true, true, false);   \
-  } else if (bf16) {                                 \
-    ADAMAS_LAUNCH_SELATT_BF(G, true, false, false);  \
-  } else if (hnd) {                                  \
-    ADAMAS_LAUNCH_SELATT_BF(G, false, true, false);  \
-  } else {                                           \
-    ADAMAS_LAUNCH_SELATT_BF(G, false, false, false); \
-  }
-  // 8 candidate slots per thread and group: the smallest group count that covers the slots
-  const uint64_t slots = static_cast<uint64_t>(w.cand_chunks) * w.cand_stride;
-  if (slots <= 4096) {
-    ADAMAS_LAUNCH_SELATT(1)
-  } else if (slots <= 8192) {
-    ADAMAS_LAUNCH_SELATT(2)
-  } else if (slots <= 12288) {
-    ADAMAS_LAUNCH_SELATT(3)
+  if (qsrc) {
+    ADAMAS_LAUNCH_SELATT_BF(false, false, true);
+  } else if (bf16 && hnd) {
+    ADAMAS_LAUNCH_SELATT_BF(true, true, false);
+  } else if (bf16) {
+    ADAMAS_LAUNCH_SELATT_BF(true, false, false);
+  } else if (hnd) {
+    ADAMAS_LAUNCH_SELATT_BF(false, true, false);
   } else {
-    ADAMAS_LAUNCH_SELATT(4)
+    ADAMAS_LAUNCH_SELATT_BF(false, false, false);
   }
-#undef ADAMAS_LAUNCH_SELATT
 #undef ADAMAS_LAUNCH_SELATT_BF
   ADAMAS_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
 
-extern "C" int adamas_step_attend_f(const void* q, const void* kv_data,
+extern "C" int adamas_step_attend_f(const void* q, const void* kv_data, const void* code_data,
                                     const int32_t* page_indices, const int32_t* page_indptr,
                                     const int32_t* seq_lens, uint32_t budget, void* out,
                                     int32_t* sel_out, void* workspace, size_t workspace_bytes,
@@ -780,22 +971,24 @@ extern "C" int adamas_step_attend_f(const void* q, const void* kv_data,
                                     uint32_t head_dim, uint32_t page_size, float sm_scale,
                                     uint32_t max_seq_len, uint32_t page_table_stride,
                                     uint32_t flags, adamas_stream_t stream) {
-  return step_attend_impl(q, const_cast<void*>(kv_data), page_indices, page_indptr, seq_lens, budget,
-                          out, sel_out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
-                          head_dim, page_size, sm_scale, max_seq_len, page_table_stride, flags,
-                          stream, nullptr, nullptr);
+  return step_attend_impl(q, const_cast<void*>(kv_data), const_cast<void*>(code_data), page_indices,
+                          page_indptr, seq_lens, budget, out, sel_out, workspace, workspace_bytes,
+                          batch, num_heads, num_kv_heads, head_dim, page_size, sm_scale, max_seq_len,
+                          page_table_stride, flags, stream, nullptr);
 }
 
-extern "C" int adamas_step_attend(const void* q, const void* kv_data, const int32_t* page_indices,
+extern "C" int adamas_step_attend(const void* q, const void* kv_data, const void* code_data,
+                                  const int32_t* page_indices,
                                   const int32_t* page_indptr, const int32_t* seq_lens,
                                   uint32_t budget, void* out, int32_t* sel_out, void* workspace,
                                   size_t workspace_bytes, uint32_t batch, uint32_t num_heads,
                                   uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size,
                                   float sm_scale, uint32_t max_seq_len, uint32_t page_table_stride,
                                   adamas_stream_t stream) {
-  return adamas_step_attend_f(q, kv_data, page_indices, page_indptr, seq_lens, budget, out, sel_out,
-                              workspace, workspace_bytes, batch, num_heads, num_kv_heads, head_dim,
-                              page_size, sm_scale, max_seq_len, page_table_stride, 0u, stream);
+  return adamas_step_attend_f(q, kv_data, code_data, page_indices, page_indptr, seq_lens, budget,
+                              out, sel_out, workspace, workspace_bytes, batch, num_heads,
+                              num_kv_heads, head_dim, page_size, sm_scale, max_seq_len,
+                              page_table_stride, 0u, stream);
 }
 
 extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const void* kv_data,
@@ -831,10 +1024,10 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
                                       num_kv_heads, page_size, max_seq_len, page_table_stride,
                                       flags, stream);
     if (rc != 0) return rc;
-    return adamas_step_attend_f(q, kv_data, page_indices, page_indptr, seq_lens, budget, out,
-                                sel_out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
-                                head_dim, page_size, sm_scale, max_seq_len, page_table_stride, flags,
-                                stream);
+    return adamas_step_attend_f(q, kv_data, code_data, page_indices, page_indptr, seq_lens, budget,
+                                out, sel_out, workspace, workspace_bytes, batch, num_heads,
+                                num_kv_heads, head_dim, page_size, sm_scale, max_seq_len,
+                                page_table_stride, flags, stream);
   }
 
   uint16_t* dist = reinterpret_cast<uint16_t*>(ws + w.dist_off);
@@ -844,22 +1037,34 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
   // histograms, then the attention over the selected tokens (three launches)
   if (n_sel > 0 && max_seq_len > 1 && max_seq_len - 1 <= 131072 && w.hist_stride > 0 &&
       batch <= 65535) {
-    const int est_heads = estimator_heads(w.hist_stride, num_heads, batch);
+    // workgroups of 4 heads wherever the 8-head ones would leave CUs idle or unevenly loaded
+    const uint64_t wide = static_cast<uint64_t>(w.hist_stride) * (num_heads / kFusedHeads) * batch;
+    const int est_heads =
+        (batch > 1 || (2 * wide + kStepWorkgroups - 1) / kStepWorkgroups <
+                          2 * ((wide + kStepWorkgroups - 1) / kStepWorkgroups))
+            ? 4
+            : kFusedHeads;
     const dim3 grid(w.hist_stride, num_heads / est_heads, batch);
+    StepGeom hist_geom;  // chunks of 512 tokens
+    hist_geom.units_q = kFusedBlock / kStepUnit;
+    hist_geom.units_r = 0;
+    hist_geom.kc = 0;
+    hist_geom.kc_log2 = 0;
     unsigned char* hist = reinterpret_cast<unsigned char*>(ws + w.hist_off);
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint32_t* rowmap = reinterpret_cast<uint32_t*>(ws + w.rowmap_off);
     int32_t* sel_rows = reinterpret_cast<int32_t*>(ws + w.rows_off);
 #define ADAMAS_LAUNCH_ESTHIST_H(PG, HEADS)                                                       \
-  hipLaunchKernelGGL((estimate_select_kernel<PG, 1, true, HEADS>), grid, dim3(HEADS * kWave), 0, \
-                     s,                                                                          \
+  hipLaunchKernelGGL((estimate_select_kernel<PG, 1, false, true, HEADS>), grid,                  \
+                     dim3(HEADS * kWave), 0, s,                                                  \
                      static_cast<const uint16_t*>(q_code),                                      \
                      static_cast<const unsigned char*>(code_data), page_indices, page_indptr,   \
-                     seq_lens, static_cast<uint64_t*>(nullptr), hist, w.hist_stride, n_sel, 0u, \
+                     seq_lens, static_cast<uint64_t*>(nullptr), hist_geom,                      \
+                     static_cast<uint16_t*>(nullptr),                                           \
                      num_heads, num_kv_heads, group_inv16(num_heads / num_kv_heads),           \
                      page_size, page_table_stride,                                              \
-                     rows_per_page_of(flags, page_size, num_kv_heads), dist,                    \
-                     static_cast<int64_t>(w.dist_stride), rowmap)
+                     rows_per_page_of(flags, page_size, num_kv_heads), hist, w.hist_stride,     \
+                     dist, static_cast<int64_t>(w.dist_stride), rowmap)
 #define ADAMAS_LAUNCH_ESTHIST(PG)        \
   if (est_heads == 4) {                  \
     ADAMAS_LAUNCH_ESTHIST_H(PG, 4);      \
@@ -942,10 +1147,10 @@ extern "C" int adamas_decode_layer_step(const void* qkv, const float* cos_table,
                                 workspace, workspace_bytes, batch, num_heads, num_kv_heads,
                                 page_size, max_seq_len, page_table_stride, 0u, stream, &src);
   if (rc != 0) return rc;
-  return step_attend_impl(nullptr, kv_data, page_indices, page_indptr, seq_lens, budget, out,
-                          sel_out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
+  return step_attend_impl(nullptr, kv_data, code_data, page_indices, page_indptr, seq_lens, budget,
+                          out, sel_out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
                           head_dim, page_size, sm_scale, max_seq_len, page_table_stride, 0u, stream,
-                          &src, code_data);
+                          &src);
 }
 
 // ---- the decode step for callers that cannot allocate ----------------------------------------------

@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F
 
 from . import utils as U
-from .utils.controller import ALL_PAST_TOKENS, InferenceController
+from .utils.controller import ALL_PAST_TOKENS, ORTHONORMAL_SCALE, InferenceController
 
 
 @dataclass
@@ -171,7 +171,7 @@ class LlamaShapedDecoder:
 
     # --- state ------------------------------------------------------------------------------------
     def init_cache(self, page_size: int, max_seq_len: int, token_budget: int, page_order=None,
-                   hadamard_scale: float = 1.0):
+                   hadamard_scale: float = ORTHONORMAL_SCALE):
         """Counterpart of Adamas_init(page_size, max_seq_len, token_budget), llama.py:520-552."""
         c = self.cfg
         self.ctrl = InferenceController(c.num_layers, c.num_heads, c.head_dim, page_size,

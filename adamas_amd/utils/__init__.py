@@ -20,7 +20,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from .controller import ALL_PAST_TOKENS, InferenceController
+from .controller import ALL_PAST_TOKENS, ORTHONORMAL_SCALE, RAW_SCALE, InferenceController
 from .paging import CODE_WORDS, KvCache, PagePool, PagedSequences, TensorLayout
 
 __all__ = [
@@ -31,6 +31,8 @@ __all__ = [
     "InferenceController",
     "BatchDecodeWithPagedKVCacheWrapper",
     "ALL_PAST_TOKENS",
+    "ORTHONORMAL_SCALE",
+    "RAW_SCALE",
     "hadamard_transform",
     "pack_2bit",
     "append_kvh",
@@ -71,12 +73,14 @@ def _check_cuda_contig(t: torch.Tensor, name: str, dtype=None, ndim=None):
         raise RuntimeError(f"{name} must have {ndim} dimensions, got {t.dim()}")
 
 
-def hadamard_transform(x: torch.Tensor, inplace: bool = False, scale: float = 1.0) -> torch.Tensor:
+def hadamard_transform(x: torch.Tensor, inplace: bool = False,
+                       scale: float = ORTHONORMAL_SCALE) -> torch.Tensor:
     """y = x . H_128 * scale over the last axis, fp32 butterfly, result in the dtype of x (fp16 or bf16).
 
     Stand-in for `faster_hadamard_transform.hadamard_transform(x, inplace)` as the reference calls it
-    (adamas/models/Adamas.py:120, :150).  `scale` 1.0 is the raw +-1 butterfly, 128**-0.5 the
-    orthonormal transform.
+    (adamas/models/Adamas.py:120, :150), which passes no scale: the default is the orthonormal
+    transform (128**-0.5) that module's published source computes; `scale` 1.0 is the raw +-1
+    butterfly.
     """
     _check_cuda_contig(x, "x", _FLOAT_DTYPES)
     if x.shape[-1] != 128:

@@ -32,12 +32,20 @@ class _AllPastTokens:
 
 ALL_PAST_TOKENS = _AllPastTokens()
 
+# Scale of the Hadamard transform behind the 2-bit codes.  The reference calls a third-party transform
+# without a scale argument (adamas/models/Adamas.py:120,150) and bucketizes the result against the
+# absolute thresholds -10 / 0 / 10 (kernels/include/decode/decode_page.cuh:385); that module's published
+# source is orthonormal (x . H_128 / sqrt(128)), so that is what a caller who passes nothing gets here.
+# 1.0 is the raw +-1 butterfly.
+ORTHONORMAL_SCALE = 128 ** -0.5
+RAW_SCALE = 1.0
+
 
 class InferenceController:
     def __init__(self, num_layers, num_heads, head_dim, page_size,
                  page_budget,   # token budget, current token included
                  max_seq_len,   # capacity of every sequence, in tokens
-                 dtype, device, *, batch_size: int = 1, hadamard_scale: float = 1.0,
+                 dtype, device, *, batch_size: int = 1, hadamard_scale: float = ORTHONORMAL_SCALE,
                  code_from_fp32: bool = False, page_order=None, num_kv_heads: Optional[int] = None,
                  layout: int = TensorLayout.NHD):
         if dtype not in (torch.float16, torch.bfloat16):

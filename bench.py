@@ -117,6 +117,10 @@ def parse_args():
     ap.add_argument("--kv-layout", choices=("nhd", "hnd"), default="nhd",
                     help="page layout of the KV cache: [2, page, heads, 128] (the reference's) or "
                          "[2, heads, page, 128]")
+    ap.add_argument("--hadamard-scale", type=float, default=1.0,
+                    help="scale of the Hadamard transform behind the codes of the timed caches: 1.0 = raw "
+                         "+-1 butterfly (all four code levels on the synthetic inputs; the headline), "
+                         "0.08838834764831845 = 128**-0.5, the orthonormal transform (the library default)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time box of the CPU baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-e2e", action="store_true",
@@ -215,7 +219,7 @@ def run_batched(args, w, lib, torch, U, _lib, dev):
     n_pages = (cap // P) * B
     order = np.random.default_rng(w.seed).permutation(n_pages).tolist()
     ctrl = U.InferenceController(n_layers, H, D, P, budget, cap, torch.float16, dev, batch_size=B,
-                                 page_order=order)
+                                 page_order=order, hadamard_scale=args.hadamard_scale)
     g = torch.Generator(device=dev).manual_seed(w.seed)
     gain = torch.ones(H, D, device=dev)
     for h in range(H):
@@ -266,9 +270,10 @@ def run_batched(args, w, lib, torch, U, _lib, dev):
 
     def k_attend(i):
         ly = i % n_layers
-        rc = lib.adamas_step_attend(q.data_ptr(), ctrl.pool.kv[ly].data_ptr(), tbl, indptr, sl,
-                                    budget, out.data_ptr(), None, ws.data_ptr(), ws.numel(), B, H, H, D,
-                                    P, sm_scale, Lmax, ctrl.seqs.max_pages, _lib.current_stream())
+        rc = lib.adamas_step_attend(q.data_ptr(), ctrl.pool.kv[ly].data_ptr(),
+                                    ctrl.pool.codes[ly].data_ptr(), tbl, indptr, sl, budget,
+                                    out.data_ptr(), None, ws.data_ptr(), ws.numel(), B, H, H, D, P,
+                                    sm_scale, Lmax, ctrl.seqs.max_pages, _lib.current_stream())
         if rc:
             _lib.check(rc, "adamas_step_attend")
 
@@ -302,7 +307,8 @@ def run_batched(args, w, lib, torch, U, _lib, dev):
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "u32 popcount on 2-bit codes + fp16 KV with fp32 softmax", "data": "synthetic",
         "config": {"workload": w.name, "batch": B, "heads": H, "head_dim": D, "seq_lens": lens,
-                   "page_size": P, "token_budget": budget, "rotated_layer_caches": n_layers,
+                   "page_size": P, "token_budget": budget, "hadamard_scale": args.hadamard_scale,
+                   "rotated_layer_caches": n_layers,
                    "timed_region": "HIP graph of K steps", "launches_per_step": 2},
         "achieved_hbm_GBps": round(step_bytes / (step_us * 1e-6) / 1e9, 1),
         "frac_of_hbm_roofline": round(step_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
@@ -391,7 +397,7 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
     fdt = torch.bfloat16 if bf16 else torch.float16
     layout = U.TensorLayout.HND if args.kv_layout == "hnd" else U.TensorLayout.NHD
     ctrl = U.InferenceController(n_layers, H, D, P, budget, L, fdt, dev, page_order=order,
-                                 num_kv_heads=Hkv, layout=layout)
+                                 num_kv_heads=Hkv, layout=layout, hadamard_scale=args.hadamard_scale)
     kv_flags = ctrl.kv_flags   # the *_f entry points with flags 0 are the plain ones
     k_dev, v_dev, q_dev = (seq.k[:, :Hkv].to(dev).to(fdt), seq.v[:, :Hkv].to(dev).to(fdt),
                            seq.q.to(dev).to(fdt))
@@ -477,9 +483,9 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
 
     def k_attend(i):
         ly = i % n_layers
-        rc = lib.adamas_step_attend_f(q3.data_ptr(), kv_ptr[ly], tbl, indptr, lens, budget,
-                                      out.data_ptr(), sel.data_ptr(), ws.data_ptr(), ws.numel(), 1,
-                                      H, Hkv, D, P, sm_scale, L, tbl_stride, kv_flags,
+        rc = lib.adamas_step_attend_f(q3.data_ptr(), kv_ptr[ly], code_ptr[ly], tbl, indptr, lens,
+                                      budget, out.data_ptr(), sel.data_ptr(), ws.data_ptr(),
+                                      ws.numel(), 1, H, Hkv, D, P, sm_scale, L, tbl_stride, kv_flags,
                                       _lib.current_stream())
         if rc:
             _lib.check(rc, "adamas_step_attend")
@@ -492,7 +498,7 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         ly = i % n_layers
         rc = lib.adamas_append_decode(q3.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), None,
                                       qc_tmp.data_ptr(), kv_ptr[ly], code_ptr[ly], tbl, indptr, lens,
-                                      1, H, Hkv, D, P, 1.0, _lib.dtype_flags(fdt),
+                                      1, H, Hkv, D, P, args.hadamard_scale, _lib.dtype_flags(fdt),
                                       _lib.current_stream())
         if rc:
             _lib.check(rc, "adamas_append_decode")
@@ -614,12 +620,12 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         torch.set_num_threads(os.cpu_count() or 1)
         hmat = P_cpu.hadamard_matrix()
         qf, kf, vf = seq.q.float(), seq.k.float(), seq.v.float()
-        P_cpu.decode_layer_step(qf, kf[:4096], vf[:4096], budget, hmat)      # warm
+        P_cpu.decode_layer_step(qf, kf[:4096], vf[:4096], budget, hmat, args.hadamard_scale)      # warm
         times = []
         t_start = time.time()
         while len(times) < 3 or (time.time() - t_start < args.cpu_seconds and len(times) < 50):
             t1 = time.perf_counter()
-            P_cpu.decode_layer_step(qf, kf, vf, budget, hmat)
+            P_cpu.decode_layer_step(qf, kf, vf, budget, hmat, args.hadamard_scale)
             times.append(time.perf_counter() - t1)
         cpu_us = float(np.median(times)) * 1e6
         cpu = {"value": round(cpu_us, 1), "unit": "us", "cores": torch.get_num_threads(),
@@ -628,12 +634,12 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
                          f"{torch.__version__} fp32 on the host, key codes recomputed every step as "
                          "the reference's PyTorch path does; median"}
         # the same with the key codes kept from step to step (what a code cache would give the CPU)
-        kc = P_cpu.codes(kf.transpose(0, 1), hmat)
+        kc = P_cpu.codes(kf.transpose(0, 1), hmat, args.hadamard_scale)
         cached = []
         t_start = time.time()
         while len(cached) < 3 or (time.time() - t_start < args.cpu_seconds / 3 and len(cached) < 50):
             t1 = time.perf_counter()
-            P_cpu.decode_layer_step(qf, kf, vf, budget, hmat, k_codes=kc)
+            P_cpu.decode_layer_step(qf, kf, vf, budget, hmat, args.hadamard_scale, k_codes=kc)
             cached.append(time.perf_counter() - t1)
         cpu["cached_codes_value"] = round(float(np.median(cached)) * 1e6, 1)
         log(f"cpu baseline: {cpu_us:.0f} us per layer-step on {cpu['cores']} threads "
@@ -657,6 +663,7 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         "config": {"workload": w.name, "batch": 1, "heads": H, "kv_heads": Hkv, "head_dim": D,
                    "kv_len": L,
                    "page_size": P, "kv_layout": args.kv_layout.upper(), "token_budget": budget,
+                   "hadamard_scale": args.hadamard_scale,
                    "rotated_layer_caches": n_layers,
                    "timed_region": "HIP graph of K steps",
                    "launches_per_step": 2 if fused else 3},

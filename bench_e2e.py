@@ -19,12 +19,13 @@ def log(msg):
 
 
 def run_e2e(prompt=32768, new_tokens=256, budget=128, page_size=16, layers=32,
-            model_name="llama2_7b", use_graph=True, log=log):
+            model_name="llama2_7b", use_graph=True, log=log, hadamard_scale=None):
     """Prefill + greedy decoding, sparse path against dense attention on every layer; returns the
     result record (protocol of the reference's scripts/bench_textgen.py:89-116: time per generated
     token after the prefill, here between device events around the whole decode loop)."""
     import torch
     from adamas_amd import _lib
+    from adamas_amd.utils import ORTHONORMAL_SCALE
     from adamas_amd.decoder import DecoderConfig, LlamaShapedDecoder
 
     if not torch.cuda.is_available():
@@ -40,10 +41,12 @@ def run_e2e(prompt=32768, new_tokens=256, budget=128, page_size=16, layers=32,
         f"({torch.cuda.memory_allocated() / 2**30:.1f} GiB allocated)")
     ids = torch.randint(0, cfg.vocab, (prompt,), generator=torch.Generator().manual_seed(5)).to(dev)
     max_len = prompt + new_tokens
+    # the codes of the caches: the library's default transform (orthonormal) unless told otherwise
+    scale = ORTHONORMAL_SCALE if hadamard_scale is None else float(hadamard_scale)
 
     results = {}
     for mode, sparse in (("adamas", True), ("dense", False)):
-        model.init_cache(page_size, max_len, budget)
+        model.init_cache(page_size, max_len, budget, hadamard_scale=scale)
         torch.cuda.synchronize()
         t0 = time.time()
         first = model.prefill(ids).argmax(-1)
@@ -68,7 +71,7 @@ def run_e2e(prompt=32768, new_tokens=256, budget=128, page_size=16, layers=32,
         "config": {"workload": f"c5_e2e_{model_name}_shape", "layers": cfg.num_layers,
                    "query_heads": cfg.num_heads, "kv_heads": cfg.kv_heads,
                    "prompt_tokens": prompt, "new_tokens": new_tokens,
-                   "token_budget": budget, "page_size": page_size,
+                   "token_budget": budget, "page_size": page_size, "hadamard_scale": scale,
                    "dense_layers": cfg.dense_layers, "decode_loop": "one HIP graph per token"
                    if use_graph else "eager"},
         "adamas": a, "dense": d,
@@ -86,9 +89,12 @@ def main():
     ap.add_argument("--model", choices=["llama2_7b", "llama3_8b"], default="llama2_7b",
                     help="shape of the random-init model (llama3_8b: 8 key/value heads)")
     ap.add_argument("--no-graph", action="store_true", help="eager decode loop (host work per step)")
+    ap.add_argument("--hadamard-scale", type=float, default=None,
+                    help="scale of the Hadamard transform behind the codes (default: 128**-0.5)")
     args = ap.parse_args()
     print(json.dumps(run_e2e(args.prompt, args.new_tokens, args.budget, args.page_size, args.layers,
-                             args.model, not args.no_graph)), flush=True)
+                             args.model, not args.no_graph, hadamard_scale=args.hadamard_scale)),
+          flush=True)
 
 
 if __name__ == "__main__":

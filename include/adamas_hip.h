@@ -294,15 +294,18 @@ int adamas_decode_step_noalloc(const void* q, const void* q_code, const void* kv
 /*
  * The two halves of adamas_decode_step, for callers that want to time or schedule them separately.
  * adamas_step_fused_supported returns 1 when these sizes are served by the two-launch path (budget
- * <= 256 and at most 16384 candidate slots per head: ceil((max_seq_len-1)/C) * roundup8(budget-1) for a
- * chunk size C of 512, 1024 or 2048 tokens, e.g. 131072 tokens at budget 256);
- * otherwise adamas_decode_step runs estimate, top-k and attention as three launches and the two
- * functions below return ADAMAS_E_UNSUPPORTED.
+ * <= 256; one sequence of up to 131072 tokens, or several whose chunk lists fit: at most 64 chunks of
+ * 512, 1024 or 2048 tokens each); otherwise adamas_decode_step runs estimate, top-k and attention as
+ * three launches and the two functions below return ADAMAS_E_UNSUPPORTED.
  *   adamas_step_candidates : distance estimate over the code cache fused with the selection of the
- *                            budget-1 nearest tokens of every chunk (written, with a
- *                            per-chunk histogram of their distances, into the workspace).
- *   adamas_step_attend     : final selection among the candidates (same tie rule) and attention over
- *                            the selected tokens plus the current one.
+ *                            nearest tokens of every chunk (chunks of a single sequence are balanced:
+ *                            their lengths differ by at most 16 tokens and their number does not
+ *                            change with the length).  Every chunk leaves a list of its nearest
+ *                            tokens per head, and the query codes, in the workspace.
+ *   adamas_step_attend     : final selection among the listed tokens (same tie rule) and attention
+ *                            over the selected tokens plus the current one.  A chunk whose list is
+ *                            used up by the selection is scored again from code_data, so the
+ *                            selection is exact for any input.
  * No counterpart in the reference: its three operators (adamas/utils/__init__.py:203-308) are one
  * launch each and exchange the full [heads, L-1] distance matrix through HBM.
  */
@@ -313,25 +316,25 @@ int adamas_step_candidates(const void* q_code, const void* code_data, const int3
                            void* workspace, size_t workspace_bytes, uint32_t batch,
                            uint32_t num_heads, uint32_t num_kv_heads, uint32_t page_size,
                            uint32_t max_seq_len, uint32_t page_table_stride, adamas_stream_t stream);
-int adamas_step_attend(const void* q, const void* kv_data, const int32_t* page_indices,
-                       const int32_t* page_indptr, const int32_t* seq_lens, uint32_t budget,
-                       void* out, int32_t* sel_out, void* workspace, size_t workspace_bytes,
-                       uint32_t batch, uint32_t num_heads, uint32_t num_kv_heads, uint32_t head_dim,
-                       uint32_t page_size, float sm_scale, uint32_t max_seq_len,
-                       uint32_t page_table_stride, adamas_stream_t stream);
+int adamas_step_attend(const void* q, const void* kv_data, const void* code_data,
+                       const int32_t* page_indices, const int32_t* page_indptr,
+                       const int32_t* seq_lens, uint32_t budget, void* out, int32_t* sel_out,
+                       void* workspace, size_t workspace_bytes, uint32_t batch, uint32_t num_heads,
+                       uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size, float sm_scale,
+                       uint32_t max_seq_len, uint32_t page_table_stride, adamas_stream_t stream);
 int adamas_step_candidates_f(const void* q_code, const void* code_data,
                              const int32_t* page_indices, const int32_t* page_indptr,
                              const int32_t* seq_lens, uint32_t budget, void* workspace,
                              size_t workspace_bytes, uint32_t batch, uint32_t num_heads,
                              uint32_t num_kv_heads, uint32_t page_size, uint32_t max_seq_len,
                              uint32_t page_table_stride, uint32_t flags, adamas_stream_t stream);
-int adamas_step_attend_f(const void* q, const void* kv_data, const int32_t* page_indices,
-                         const int32_t* page_indptr, const int32_t* seq_lens, uint32_t budget,
-                         void* out, int32_t* sel_out, void* workspace, size_t workspace_bytes,
-                         uint32_t batch, uint32_t num_heads, uint32_t num_kv_heads,
-                         uint32_t head_dim, uint32_t page_size, float sm_scale,
-                         uint32_t max_seq_len, uint32_t page_table_stride, uint32_t flags,
-                         adamas_stream_t stream);
+int adamas_step_attend_f(const void* q, const void* kv_data, const void* code_data,
+                         const int32_t* page_indices, const int32_t* page_indptr,
+                         const int32_t* seq_lens, uint32_t budget, void* out, int32_t* sel_out,
+                         void* workspace, size_t workspace_bytes, uint32_t batch,
+                         uint32_t num_heads, uint32_t num_kv_heads, uint32_t head_dim,
+                         uint32_t page_size, float sm_scale, uint32_t max_seq_len,
+                         uint32_t page_table_stride, uint32_t flags, adamas_stream_t stream);
 
 /*
  * Per-token operators of the decoder around the attention path, one launch each (fp16 in/out, fp32

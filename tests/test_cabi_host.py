@@ -94,7 +94,7 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.adamas_step_fused_supported(1, 32, 4096, 1024) == 0        # budget beyond 256
     assert lib.adamas_step_candidates(16, 16, 16, 16, 16, 1024, 256, 1 << 30, 1, 32, 32, 16, 4096, 0, None) == -2
     assert lib.adamas_step_candidates(16, 16, 16, None, 16, 128, 256, 1 << 30, 1, 32, 32, 16, 4096, 0, None) == -1
-    assert lib.adamas_step_attend(16, 16, 16, 16, 16, 128, 16, None, None, 0, 1, 32, 32, 128, 16, 0.1, 4096, 0, None) == -1
+    assert lib.adamas_step_attend(16, 16, 16, 16, 16, 16, 128, 16, None, None, 0, 1, 32, 32, 128, 16, 0.1, 4096, 0, None) == -1
     assert "workspace" in _lib.error_string(-3)
     with pytest.raises(RuntimeError):
         _lib.check(-2, "x")

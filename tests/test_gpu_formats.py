@@ -101,7 +101,7 @@ def test_step_formats(gpu_device, L, hq, hkv, page_size, budget, fused_append, d
     if fused_append:
         q_code = U.append_kvh(kd[L - 1:], vd[L - 1:], None, ctrl, 0, q=qd[None])
     else:
-        h = U.hadamard_transform(torch.cat((qd, kd[L - 1])).contiguous())     # [Hq + Hkv, D]
+        h = U.hadamard_transform(torch.cat((qd, kd[L - 1])).contiguous(), scale=ctrl.hadamard_scale)     # [Hq + Hkv, D]
         if hq == hkv:
             h = h.view(2, hq, 128)
         q_code = U.append_kvh(kd[L - 1:], vd[L - 1:], h, ctrl, 0)

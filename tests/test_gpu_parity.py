@@ -467,6 +467,86 @@ def test_step_random_shapes_match_three_launch_path(gpu_device, kv_len, budget, 
     assert np.abs(T.np16(o).astype(np.float64) - T.np16(o_f).astype(np.float64)).max() <= ATTN_TOL
 
 
+def _device_sequence(gpu_device, kv_len, seed, kind="random"):
+    """q [32, 128], k, v [L, 32, 128] fp16 drawn on the device (long sequences without the host
+    generator's seconds per test); same distribution as synth.make_sequence, no needles.
+    kind "equal": every key equals key 0 (all distances tied: the selection is the first tokens,
+    which the stable argsort in _assert_step_equals_operators restates);
+    kind "clustered": the last 700 tokens are noisy copies of the query (one chunk holds most of the
+    selection, with distinct distances); kind "runs": keys repeat in runs of 300 tokens drawn from 5
+    rows (long runs of equal distances across chunk boundaries)."""
+    g = torch.Generator(device=gpu_device).manual_seed(seed)
+    gain = torch.ones(32, 128, device=gpu_device)
+    for h in range(32):
+        gain[h, torch.randperm(128, generator=g, device=gpu_device)[:4]] = 8.0
+    q = (torch.randn(32, 128, generator=g, device=gpu_device) * gain).half()
+    k = (torch.randn(kv_len, 32, 128, generator=g, device=gpu_device) * gain).half()
+    v = torch.randn(kv_len, 32, 128, generator=g, device=gpu_device).half()
+    if kind == "equal":
+        k = k[:1].expand(kv_len, 32, 128).contiguous()
+    elif kind == "clustered":
+        m = min(700, kv_len - 1)
+        noise = torch.randn(m, 32, 128, generator=g, device=gpu_device) * gain
+        mix = torch.rand(m, 1, 1, generator=g, device=gpu_device) * 0.6 + 0.2
+        k[kv_len - 1 - m:kv_len - 1] = (q.float()[None] * mix + noise * (1 - mix)).half()
+    elif kind == "runs":
+        pick = (torch.arange(kv_len, device=gpu_device) // 300) % 5
+        k = k[:5][pick].contiguous()
+    return synth.SequenceData(q=q, k=k, v=v, needles=None)
+
+
+def _assert_step_equals_operators(gpu_device, seq, budget, page_size, shuffle_seed=5, scale=1.0):
+    """The two-launch step against the three stand-alone operators (pinned to the oracle by the
+    tests above): identical index sets, every entry a distinct past token, outputs within tolerance;
+    and the operators' own selection against a stable argsort of the distances they selected from."""
+    _, q_code, est, sel, o, o_f, sel_f = _run_step(gpu_device, seq, budget, page_size, shuffle_seed,
+                                                   scale=scale)
+    a = np.sort(T.np16(sel).astype(np.int64), axis=1)
+    b = np.sort(T.np16(sel_f).astype(np.int64), axis=1)
+    d = T.np16(est).astype(np.int64)
+    d = d.reshape(-1, d.shape[-1])
+    for h in (0, 7, 31):
+        want = np.sort(np.argsort(d[h], kind="stable")[:budget - 1])
+        assert np.array_equal(a[h], want), h
+    assert np.array_equal(a, b)
+    assert (a >= 0).all() and (np.diff(a, axis=1) > 0).all()
+    assert np.abs(T.np16(o).astype(np.float64) - T.np16(o_f).astype(np.float64)).max() <= ATTN_TOL
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("kv_len", [
+    16384, 16385, 16400, 24000,          # narrow workgroups: 32 balanced chunks
+    32768, 32769, 32770, 32784, 32785,   # 64 chunks of 512 tokens, then of 512 and 528
+    33024, 33025, 36864, 40960, 40961,   # ... 576, 640 and 656 tokens
+    49152, 49153, 65536, 65537, 65553,   # two whole passes, three partial ones
+    98304, 98321, 131072,                # three and four passes
+    513, 1025, 8191, 8192, 8193, 16383,  # chunks of 512 tokens that do not fill the chip
+])
+def test_step_balanced_chunks_at_length_boundaries(gpu_device, kv_len):
+    """Lengths on both sides of every boundary of the chunk plan (the number of passes a workgroup
+    makes, a partial last pass, the heads per workgroup, the last unit of a chunk)."""
+    assert _lib.load().adamas_step_fused_supported(1, 32, kv_len, 128) == 1
+    T.heartbeat(f"balanced chunks: L={kv_len}")
+    seq = _device_sequence(gpu_device, kv_len, kv_len)
+    _assert_step_equals_operators(gpu_device, seq, 128, 16)
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("scale", SCALES)
+@pytest.mark.parametrize("kind", ["equal", "clustered", "runs"])
+@pytest.mark.parametrize("kv_len,budget,page_size", [
+    (33000, 128, 16), (32768, 128, 16), (70000, 256, 16), (5000, 64, 3), (131072, 256, 16),
+    (20000, 17, 16), (40000, 128, 1),
+])
+def test_step_truncated_chunk_lists_are_rescored(gpu_device, kv_len, budget, page_size, kind, scale):
+    """Inputs whose selection needs more tokens of one chunk than the chunk's list holds: every
+    distance tied, most of the selection inside one chunk, long runs of equal distances.  The second
+    launch scores such chunks again, and the result stays exact."""
+    T.heartbeat(f"truncated lists: L={kv_len} budget={budget} {kind}")
+    seq = _device_sequence(gpu_device, kv_len, kv_len + budget, kind)
+    _assert_step_equals_operators(gpu_device, seq, budget, page_size, scale=scale)
+
+
 @pytest.mark.timeout(900)
 @pytest.mark.parametrize("kv_len,budget,page_size", [
     (5000, 300, 16), (20000, 512, 16), (32768, 1024, 16), (9000, 4096, 3), (40000, 2048, 1),
@@ -727,7 +807,7 @@ def test_grouped_query_attention_step(gpu_device, hq, hkv, page_size, budget, fu
     if fused_append:
         q_code = U.append_kvh(kd[L - 1:], vd[L - 1:], None, ctrl, 0, q=qd[None])
     else:
-        h = U.hadamard_transform(torch.cat((qd, kd[L - 1])).contiguous())     # [Hq + Hkv, D]
+        h = U.hadamard_transform(torch.cat((qd, kd[L - 1])).contiguous(), scale=ctrl.hadamard_scale)     # [Hq + Hkv, D]
         if hq == hkv:
             h = h.view(2, hq, 128)    # the reference's shape for equal head counts
         q_code = U.append_kvh(kd[L - 1:], vd[L - 1:], h, ctrl, 0)
