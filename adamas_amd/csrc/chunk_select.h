@@ -244,20 +244,27 @@ __device__ __forceinline__ WavePlan wave_plan_from_hist(const uint32_t* hist_lds
 }
 
 // One wave: the kc smallest of its 64 x kItems keys (lane l holds items kItems*l .. kItems*l +
-// kItems-1 in index order; any value above 511 = no item), ties to the lowest index, written to the
-// chunk's candidate list dst[kc] as (key << 48) | (item index << 32) | payload, first the keys below
-// the chunk's threshold, then the tied ones, each class in ascending index order; unused slots are
-// filled with kEmptyCand64.  A list is a prefix of the chunk in (key, index) order: when its last
-// entry is not among the keys a caller finally selects, no key of the chunk outside the list can be.
-// hist_lds: kChunkHistWords words of LDS owned by this wave, 16-byte aligned.  payload(item, i) ->
-// 32 bits stored with the candidate, evaluated for listed items only.
+// kItems-1 in index order, kItems <= 32; any value above 511 = no item), ties to the lowest index,
+// written to the chunk's candidate list dst[kc] as (key << 48) | (item index << 32) | payload, first
+// the keys below the chunk's threshold, then the tied ones, each class in ascending index order;
+// unused slots are filled with kEmptyCand64.  A list is a prefix of the chunk in (key, index) order:
+// when its last entry is not among the keys a caller finally selects, no key of the chunk outside the
+// list can be.
+// hist_lds: kChunkHistWords words of LDS owned by this wave, 16-byte aligned.  key_of(item) -> the
+// key of an item (the caller's LDS copy: a listed item is picked by a run-time index), payload(item)
+// -> 32 bits stored with the candidate; both are evaluated for listed items only.
+// A list has a handful of entries among hundreds of items, so the items are not tested one by one
+// when the list is written: every lane walks the set bits of its own class masks, and the wave makes
+// as many rounds as its busiest lane has listed items (one or two, against kItems tests of a dozen
+// instructions each).
 // kSkipInvalid: items that are no keys are left out of the counting by a branch (worth it where many
 // lanes hold none: they would all add to one spare word); otherwise they count into a spare word
 // without a branch.
-template <int kItems, bool kSkipInvalid, typename Payload>
+template <int kItems, bool kSkipInvalid, typename KeyOf, typename Payload>
 __device__ __forceinline__ void chunk_select_capped(const uint32_t (&keys)[kItems], uint32_t kc,
                                                     uint64_t* dst, uint32_t* hist_lds,
-                                                    Payload&& payload) {
+                                                    KeyOf&& key_of, Payload&& payload) {
+  static_assert(kItems <= 32, "one class bit per item");
   const int lane = lane_id();
   *reinterpret_cast<uint4*>(&hist_lds[8 * lane]) = make_uint4(0u, 0u, 0u, 0u);
   *reinterpret_cast<uint4*>(&hist_lds[8 * lane + 4]) = make_uint4(0u, 0u, 0u, 0u);
@@ -271,16 +278,33 @@ __device__ __forceinline__ void chunk_select_capped(const uint32_t (&keys)[kItem
   }
   // the LDS operations of one wave are carried out in order: the counts are complete here
   const WavePlan p = wave_plan_from_hist(hist_lds, kc);
-  uint32_t below[kItems / 4], equal[kItems / 4];
-  raw_class_masks<kItems>(keys, p.thr, below, equal);
-  uint32_t total;
-  const uint32_t excl = lane_scan<kItems / 4>(below, equal, total);
-  lane_emit<kItems / 4>(below, equal, p.n_below, p.quota, excl & 0xffffu, excl >> 16,
-                        [&](uint32_t pos, int i) __attribute__((always_inline)) {
-                          const uint32_t tok = static_cast<uint32_t>(lane) * kItems + i;
-                          dst[pos] =
-                              (static_cast<uint64_t>((keys[i] << 16) | tok) << 32) | payload(tok, i);
-                        });
+  uint32_t below = 0, equal = 0;  // bit i: item i is below / equal to the threshold
+#pragma unroll
+  for (int i = 0; i < kItems; ++i) {
+    below |= keys[i] < p.thr ? (1u << i) : 0u;  // an empty item compares above everything
+    equal |= keys[i] == p.thr ? (1u << i) : 0u;
+  }
+  const uint32_t mine = static_cast<uint32_t>(__builtin_popcount(below)) |
+                        (static_cast<uint32_t>(__builtin_popcount(equal)) << 16);
+  const uint32_t excl = wave_inclusive_scan_dpp(mine) - mine;
+  uint32_t pb = excl & 0xffffu, pe = excl >> 16;  // items of each class in the lower lanes
+  uint32_t todo = below | (pe < p.quota ? equal : 0u);
+  while (todo) {
+    const uint32_t i = static_cast<uint32_t>(__builtin_ctz(todo));
+    todo &= todo - 1u;
+    const bool is_b = ((below >> i) & 1u) != 0;
+    const uint32_t item = static_cast<uint32_t>(lane) * kItems + i;
+    uint32_t pos, key;
+    if (is_b) {
+      pos = pb++;
+      key = key_of(item);
+    } else {  // a tied item inside the quota
+      pos = p.n_below + pe++;
+      key = p.thr;
+      if (pe >= p.quota) todo &= below;  // the quota is used up: the lane's further ties stay out
+    }
+    dst[pos] = (static_cast<uint64_t>((key << 16) | item) << 32) | payload(item);
+  }
   for (uint32_t i = p.n_take + lane; i < kc; i += kWave) dst[i] = kEmptyCand64;
 }
 

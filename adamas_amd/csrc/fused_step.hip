@@ -226,6 +226,7 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
   {
     const uint32_t head = hg * kHeads + hl;
     QueryPlanes qp;
+    uint4 qraw_copy = make_uint4(0u, 0u, 0u, 0u);
     WaveRopeLoads qload;  // kFromQkv: the query row of head hg*kHeads + wave and its rotary factors
     if (kFromQkv) {
       // issued ahead of the code loads, used after them: the wait for these leaves the code loads in flight
@@ -237,9 +238,7 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
       const uint4 qraw = *reinterpret_cast<const uint4*>(
           q_code + (static_cast<size_t>(b) * num_heads + head) * kCodeWords + half * 8u);
       qp = make_query_planes(qraw);
-      if (!kHist && chunk == 0 && sub == 0)
-        *reinterpret_cast<uint4*>(qcode_out + (static_cast<size_t>(b) * num_heads + head) * kCodeWords +
-                                  half * 8u) = qraw;
+      qraw_copy = qraw;
     }
 
     // grouped-query attention: query head h scores the codes of key head h / group; the lanes of a
@@ -300,6 +299,11 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     };
     uint4 buf0[16], buf1[16];
     issue(0, buf0);
+    // the query codes for the second launch (behind the code loads: the store waits for the query
+    // code, which must not hold the code loads back)
+    if (!kFromQkv && !kHist && chunk == 0 && sub == 0)
+      *reinterpret_cast<uint4*>(qcode_out + (static_cast<size_t>(b) * num_heads + head) * kCodeWords +
+                                half * 8u) = qraw_copy;
     if (kFromQkv) {
       float qx0, qx1;
       wave_rope_apply(qload, lane, qx0, qx1);
@@ -377,10 +381,10 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
     }
   }
   // the K row of a listed token is read when it is written out (a handful per wave)
-  chunk_select_capped<kItems, kPartial>(keys, geom.kc, dst, sh.hist[wave],
-                                        [&](uint32_t tok, int) __attribute__((always_inline)) {
-                                          return sh.krow[tok];
-                                        });
+  chunk_select_capped<kItems, kPartial>(
+      keys, geom.kc, dst, sh.hist[wave],
+      [&](uint32_t tok) __attribute__((always_inline)) -> uint32_t { return sh.dist[wave][tok]; },
+      [&](uint32_t tok) __attribute__((always_inline)) -> uint32_t { return sh.krow[tok]; });
 }
 
 // Up to 128 rows (one round of loads) the attention of launch 2 runs on the first four waves only (16
@@ -443,7 +447,15 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   const uint32_t n_slots = n_chunks << geom.kc_log2;
   const uint64_t* crow = cand + static_cast<size_t>(bh) * n_slots;
 
-  // K row of the current token: a chain of three dependent scalar loads, started first so that it
+  // ---- the candidates of this head: two slots per thread --------------------------------------------
+  // (asked for ahead of everything that waits for the sequence length: the list of a sequence
+  // without tokens is valid memory, if meaningless)
+  const uint32_t slot0 = 2u * tid;
+  const bool have = slot0 < n_slots;
+  uint4 raw = make_uint4(~0u, ~0u, ~0u, ~0u);  // an unused slot is all ones
+  if (have) raw = *reinterpret_cast<const uint4*>(crow + slot0);  // lists are 64-byte aligned
+
+  // K row of the current token: a chain of three dependent scalar loads, started early so that it
   // has long finished when the row list is closed
   const int32_t seq_len = seq_lens[b];
   if (seq_len <= 0) {  // a sequence without tokens: zeros and an empty selection (whole workgroup leaves)
@@ -465,11 +477,6 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     cur_row = static_cast<int32_t>(cur_page * rows_per_page + cur_slot);
   }
 
-  // ---- the candidates of this head: two slots per thread --------------------------------------------
-  const uint32_t slot0 = 2u * tid;
-  const bool have = slot0 < n_slots;
-  uint4 raw = make_uint4(~0u, ~0u, ~0u, ~0u);  // an unused slot is all ones
-  if (have) raw = *reinterpret_cast<const uint4*>(crow + slot0);  // lists are 64-byte aligned
   sh.hist[tid] = 0u;
   if (tid < kStepMaxChunks) sh.flag[tid] = 0u;
   if (tid == 0) sh.any_flag = 0u;

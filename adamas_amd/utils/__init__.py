@@ -207,9 +207,12 @@ def decode_estimate(q: torch.Tensor, iController: InferenceController, layer_idx
     out = buf[:, :, :lmax - 1]
     if c.batch_size == 1:
         out = out[0]
-    # the controller remembers the buffer it handed out: decode_topk takes the single-pass integer
-    # selection for any view of it (slices, reshapes), whatever the caller did to the tensor object
-    c._estimate_storage = (buf.untyped_storage().data_ptr(), buf.untyped_storage().nbytes())
+    # The controller keeps the buffer it handed out (until the next estimate): decode_topk takes the
+    # single-pass integer selection for any view of it (slices, reshapes).  Holding the tensor keeps
+    # its address from being handed to another tensor by the allocator, and its version counter
+    # tells an in-place edit by the caller (est.mul_(...)) from the values the kernel wrote.
+    c._estimate_buf = buf
+    c._estimate_version = buf._version
     return out
 
 
@@ -222,7 +225,9 @@ def decode_topk(estimated_attn_score: torch.Tensor, iController: InferenceContro
     integer_keys: True promises that every estimate is an integer in [0, 511] (what decode_estimate
     produces) and selects with one histogram pass; False takes the selection for arbitrary fp16
     keys.  None (the reference's two-argument call) decides by whether the tensor is a view of the
-    buffer the controller's last decode_estimate filled; a copy of it is treated as arbitrary keys.
+    buffer the controller's last decode_estimate filled and that buffer has not been edited in
+    place since (the controller holds the buffer, so its memory cannot be reused by another tensor
+    meanwhile); a copy of it, or any other tensor, is treated as arbitrary keys.
     """
     c = iController
     est = estimated_attn_score
@@ -245,8 +250,11 @@ def decode_topk(estimated_attn_score: torch.Tensor, iController: InferenceContro
         # reference check CHECK_GE(num_pages, page_budget) in adamas/ops/csrc/topk.cu:26
         raise RuntimeError("fewer candidates than the budget")
     if integer_keys is None:
-        base, nbytes = getattr(c, "_estimate_storage", (0, 0))
-        integer_keys = nbytes > 0 and base <= est.data_ptr() < base + nbytes
+        buf = getattr(c, "_estimate_buf", None)
+        integer_keys = False
+        if buf is not None and buf._version == c._estimate_version:
+            base, nbytes = buf.untyped_storage().data_ptr(), buf.untyped_storage().nbytes()
+            integer_keys = base <= est.data_ptr() < base + nbytes
     mode = _lib.KEY_FP16_INT if integer_keys else _lib.KEY_FP16_GENERIC
     ragged = c.batch_size > 1
     buf = c.topk_workspace(n, k)

@@ -266,7 +266,8 @@ def test_rope_append_decode_equals_rope_split_plus_append(gpu_device):
     ([33000], 32, 32, 16, 128),          # 65 chunks: one more than the chip has CUs per head group
     ([9000], 32, 32, 1, 200),            # page size 1
 ])
-def test_layer_step_equals_append_then_step(gpu_device, lens, hq, hkv, page_size, budget):
+@pytest.mark.parametrize("scale", [1.0, 128 ** -0.5])
+def test_layer_step_equals_append_then_step(gpu_device, lens, hq, hkv, page_size, budget, scale):
     """adamas_decode_layer_step (query code, rotary embedding, append and step in two launches)
     against rope_append_decode + decode_step: same cache contents and codes bit for bit, same
     selections, outputs equal up to the order of the softmax accumulation."""
@@ -285,7 +286,7 @@ def test_layer_step_equals_append_then_step(gpu_device, lens, hq, hkv, page_size
     results = []
     for fused in (False, True):
         ctrl = T.make_controller(gpu_device, cap, budget, page_size, batch_size=B, shuffle_seed=3,
-                                 num_heads=hq, num_kv_heads=hkv)
+                                 num_heads=hq, num_kv_heads=hkv, scale=scale)
         for b, (kk, vv) in enumerate(past):
             if kk.shape[0]:
                 T.fill_sequence(ctrl, kk, vv, seq_idx=b)

@@ -88,12 +88,13 @@ def _make(L, hq, hkv, seed, dtype=BF):
     (5000, 32, 32, 1, 5000, True, FP, HND),
     (3000, 32, 2, 3, 2000, True, FP, HND),      # 16 query heads per key/value head
 ])
-def test_step_formats(gpu_device, L, hq, hkv, page_size, budget, fused_append, dtype, layout):
+@pytest.mark.parametrize("scale", [1.0, 128 ** -0.5])
+def test_step_formats(gpu_device, L, hq, hkv, page_size, budget, fused_append, dtype, layout, scale):
     g = hq // hkv
     bf = dtype == BF
     q, k, v = _make(L, hq, hkv, L + hq + page_size, dtype)
     ctrl = T.make_controller(gpu_device, L, budget, page_size, shuffle_seed=3, num_heads=hq,
-                             num_kv_heads=hkv, dtype=dtype, layout=layout)
+                             num_kv_heads=hkv, dtype=dtype, layout=layout, scale=scale)
     kd, vd, qd = k.to(gpu_device), v.to(gpu_device), q.to(gpu_device)
     T.fill_sequence(ctrl, kd[:L - 1], vd[:L - 1], fused=fused_append, chunk=4096)
     ctrl.prepare_hadamard(1)
@@ -107,7 +108,7 @@ def test_step_formats(gpu_device, L, hq, hkv, page_size, budget, fused_append, d
         q_code = U.append_kvh(kd[L - 1:], vd[L - 1:], h, ctrl, 0)
     k_back, v_back, codes_back = T.read_logical_cache(ctrl)
     assert np.array_equal(k_back, T.np16(k)) and np.array_equal(v_back, T.np16(v))
-    assert np.array_equal(codes_back, O.codes_from_raw(T.np16(k), bf16=bf))
+    assert np.array_equal(codes_back, O.codes_from_raw(T.np16(k), scale, bf16=bf))
 
     k_full, v_full = k.repeat_interleave(g, dim=1), v.repeat_interleave(g, dim=1)
     want_dense = O.dense_attention(T.np16(q), T.np16(k_full), T.np16(v_full))
@@ -118,7 +119,7 @@ def test_step_formats(gpu_device, L, hq, hkv, page_size, budget, fused_append, d
         assert _close(o_f[0], want_dense)
         return
 
-    ora = T.oracle_step(q, k_full, v_full, budget, bf16=bf)
+    ora = T.oracle_step(q, k_full, v_full, budget, scale=scale, bf16=bf)
     assert np.array_equal(T.words_u16(q_code)[0], ora["q_words"])
     est = U.decode_estimate(q_code, ctrl, 0)
     assert np.array_equal(T.np16(est).astype(np.int32), ora["dist"])

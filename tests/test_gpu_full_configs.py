@@ -96,7 +96,8 @@ def test_ragged_batch_of_16_at_full_size(gpu_device, scale):
 
 
 @pytest.mark.timeout(1200)
-def test_llama2_7b_shape_32k_prompt_graph_eager_and_oracle(gpu_device):
+@pytest.mark.parametrize("scale", [128 ** -0.5, 1.0])
+def test_llama2_7b_shape_32k_prompt_graph_eager_and_oracle(gpu_device, scale):
     cfg = DecoderConfig.llama2_7b()
     prompt, budget, steps = 32768, 128, 16
     T.heartbeat("7B shape: drawing weights")
@@ -105,7 +106,8 @@ def test_llama2_7b_shape_32k_prompt_graph_eager_and_oracle(gpu_device):
     outs = []
     for use_graph in (False, True):
         T.heartbeat(f"7B shape: prefill, graph={use_graph}")
-        model.init_cache(page_size=16, max_seq_len=prompt + 64, token_budget=budget)
+        model.init_cache(page_size=16, max_seq_len=prompt + 64, token_budget=budget,
+                         hadamard_scale=scale)
         first = model.prefill(ids).argmax(-1)
         T.heartbeat("7B shape: decoding")
         toks, _ = model.generate(first, steps, sparse=True, use_graph=use_graph)
@@ -138,14 +140,14 @@ def test_llama2_7b_shape_32k_prompt_graph_eager_and_oracle(gpu_device):
     k_log, v_log, words = T.read_logical_cache(ctrl, layer)
     L = k_log.shape[0]
     assert L == prompt + steps + 1
-    ora = O.decode_step(T.np16(q_rot)[0], k_log, v_log, budget, k_words=words)
+    ora = O.decode_step(T.np16(q_rot)[0], k_log, v_log, budget, scale=scale, k_words=words)
     assert np.array_equal(T.words_u16(q_code)[0], ora["q_words"])
     ok, h = T.sets_equal(T.np16(sel_a), ora["sets"], L)
     assert ok, h
     assert np.abs(T.np16(o_a)[0].astype(np.float64) - ora["out"]).max() <= ATTN_TOL
     # and the cached codes are the codes of the cached keys
     some = np.random.default_rng(0).choice(L, 512, replace=False)
-    assert np.array_equal(words[some], O.codes_from_raw(k_log[some]))
+    assert np.array_equal(words[some], O.codes_from_raw(k_log[some], scale))
     model.clear()
 
 
@@ -208,3 +210,40 @@ def test_decode_topk_integer_selection_survives_views_and_copies(gpu_device):
         assert np.array_equal(got, want)
     U.decode_topk(est.clone(), ctrl, integer_keys=True)     # the explicit promise
     assert np.array_equal(np.sort(T.np16(ctrl.topk_dindices_buffer).astype(np.int64), axis=1), want)
+
+
+def test_decode_topk_takes_arbitrary_keys_for_tensors_it_did_not_fill(gpu_device):
+    """Scores that are not the controller's own estimate (another tensor of the same shape made after
+    the caller dropped the estimate, or the estimate edited in place) hold arbitrary fp16 values:
+    decode_topk must select by value, not truncate them to integer distances."""
+    L, budget = 5000, 64
+    seq = synth.make_sequence(L, 4, torch.Generator().manual_seed(13))
+    ctrl = T.make_controller(gpu_device, L, budget, 16)
+    T.fill_sequence(ctrl, seq.k[:-1].to(gpu_device), seq.v[:-1].to(gpu_device))
+    q_code = T.decode_append(ctrl, seq.q[None].to(gpu_device), seq.k[-1:].to(gpu_device),
+                             seq.v[-1:].to(gpu_device))
+
+    def picked():
+        return np.sort(T.np16(ctrl.topk_dindices_buffer).astype(np.int64), axis=1)
+
+    def stable_smallest(scores):
+        return np.sort(np.argsort(scores.astype(np.float64), axis=1, kind="stable")[:, :budget - 1], axis=1)
+
+    est = U.decode_estimate(q_code, ctrl, 0)
+    shape = est.shape
+    del est
+    torch.cuda.synchronize()
+    # fractional and negative scores of the same shape: the allocator may well reuse the block
+    g = torch.Generator(device=gpu_device).manual_seed(1)
+    other = (torch.rand(shape, generator=g, device=gpu_device) * 3 - 1).half()
+    U.decode_topk(other, ctrl)
+    assert np.array_equal(picked(), stable_smallest(T.np16(other)))
+    # the estimate itself, scaled in place: values are no longer the integers the kernel wrote
+    est = U.decode_estimate(q_code, ctrl, 0)
+    est.mul_(0.001)
+    U.decode_topk(est, ctrl)
+    assert np.array_equal(picked(), stable_smallest(T.np16(est)))
+    # and an untouched estimate still takes the integer selection (same result as by value)
+    est = U.decode_estimate(q_code, ctrl, 0)
+    U.decode_topk(est, ctrl)
+    assert np.array_equal(picked(), stable_smallest(T.np16(est)))

@@ -789,7 +789,8 @@ def test_empty_and_single_token_sequences_through_the_c_abi(gpu_device):
     (32, 8, 16, 96), (64, 16, 16, 96), (32, 32, 16, 96), (32, 4, 3, 96), (32, 16, 16, 96),
     (64, 8, 7, 96), (32, 8, 16, 400), (64, 16, 5, 1000)])
 @pytest.mark.parametrize("fused_append", [True, False])
-def test_grouped_query_attention_step(gpu_device, hq, hkv, page_size, budget, fused_append):
+@pytest.mark.parametrize("scale", SCALES)
+def test_grouped_query_attention_step(gpu_device, hq, hkv, page_size, budget, fused_append, scale):
     """Grouped-query attention (no counterpart in the reference): the oracle is the plain one on
     K and V with every key/value head repeated for the query heads of its group.  Budgets up to
     256 run as two launches, larger ones as three (histogram mode)."""
@@ -799,7 +800,7 @@ def test_grouped_query_attention_step(gpu_device, hq, hkv, page_size, budget, fu
     k = (torch.randn(L, hkv, 128, generator=gen) * 2).half()
     v = torch.randn(L, hkv, 128, generator=gen).half()
     ctrl = T.make_controller(gpu_device, L, budget, page_size, shuffle_seed=5, num_heads=hq,
-                             num_kv_heads=hkv)
+                             num_kv_heads=hkv, scale=scale)
     kd, vd, qd = k.to(gpu_device), v.to(gpu_device), q.to(gpu_device)
     T.fill_sequence(ctrl, kd[:L - 1], vd[:L - 1])
     ctrl.prepare_hadamard(1)
@@ -814,10 +815,10 @@ def test_grouped_query_attention_step(gpu_device, hq, hkv, page_size, budget, fu
     k_back, v_back, codes_back = T.read_logical_cache(ctrl)
     assert np.array_equal(k_back.view(np.uint16), T.np16(k).view(np.uint16))
     assert np.array_equal(v_back.view(np.uint16), T.np16(v).view(np.uint16))
-    assert np.array_equal(codes_back, O.codes_from_raw(T.np16(k)))
+    assert np.array_equal(codes_back, O.codes_from_raw(T.np16(k), scale))
 
     k_full, v_full = k.repeat_interleave(g, dim=1), v.repeat_interleave(g, dim=1)
-    ora = T.oracle_step(q, k_full, v_full, budget)
+    ora = T.oracle_step(q, k_full, v_full, budget, scale=scale)
     assert np.array_equal(T.words_u16(q_code)[0], ora["q_words"])
     est = U.decode_estimate(q_code, ctrl, 0)
     assert np.array_equal(T.np16(est).astype(np.int32), ora["dist"])
