@@ -43,6 +43,7 @@ _SIGNATURES = {
                                     c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float,
                                     c_uint32, c_uint32, c_void_p]),
     "adamas_step_fused_supported": (c_int, [c_uint32, c_uint32, c_uint32, c_uint32]),
+    "adamas_step_plan": (c_int, [c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "adamas_decode_step_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32,
                                             c_uint32, c_uint32, c_uint32, c_float, c_uint32, c_uint32,
@@ -117,6 +118,15 @@ def load() -> ctypes.CDLL:
         fn.argtypes = argtypes
     _lib = lib
     return lib
+
+
+def step_plan(batch: int, num_heads: int, max_seq_len: int, budget: int) -> dict:
+    """The geometry of the two-launch decode step for these sizes (adamas_step_plan)."""
+    out = (c_uint32 * 8)()
+    check(load().adamas_step_plan(batch, num_heads, max_seq_len, budget, ctypes.addressof(out)),
+          "adamas_step_plan")
+    keys = ("ok", "heads", "chunks", "units_q", "units_r", "passes", "partial", "kc")
+    return dict(zip(keys, (int(v) for v in out)))
 
 
 def error_string(code: int) -> str:

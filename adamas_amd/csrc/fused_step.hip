@@ -781,6 +781,17 @@ extern "C" int adamas_step_fused_supported(uint32_t batch, uint32_t num_heads,
   return fused_eligible(workspace_layout(batch, num_heads, max_seq_len, budget)) ? 1 : 0;
 }
 
+extern "C" int adamas_step_plan(uint32_t batch, uint32_t num_heads, uint32_t max_seq_len,
+                                uint32_t budget, uint32_t* plan_out) {
+  if (!plan_out) return ADAMAS_E_BADARG;
+  const StepPlan p = (batch && num_heads && num_heads % 32 == 0)
+                         ? step_plan(batch, num_heads, max_seq_len, budget)
+                         : StepPlan{};
+  const uint32_t v[8] = {p.ok, p.heads, p.chunks, p.units_q, p.units_r, p.passes, p.partial, p.kc};
+  for (int i = 0; i < 8; ++i) plan_out[i] = v[i];
+  return 0;
+}
+
 // rows per page of the KV layout the K row indices are meant for
 static uint32_t rows_per_page_of(uint32_t flags, uint32_t page_size, uint32_t num_kv_heads) {
   return make_kv_layout((flags & ADAMAS_F_HND) != 0, page_size, num_kv_heads).rows_per_page;

@@ -36,15 +36,42 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 PROFILE_TRAFFIC_MD = os.path.join(ROOT, "profiles", "decode_step_kernels_c2_32k_b128.md")
 
 
+def strip_c_comments(text: str) -> str:
+    """C/C++ source without comments and without runs of white space (string and character
+    literals are kept as they are)."""
+    out = []
+    i, n = 0, len(text)
+    while i < n:
+        c = text[i]
+        if c in "\"'":                              # literal: copy to the closing quote
+            j = i + 1
+            while j < n and text[j] != c:
+                j += 2 if text[j] == "\\" else 1
+            out.append(text[i:j + 1])
+            i = j + 1
+        elif text.startswith("//", i):
+            j = text.find("\n", i)
+            i = n if j < 0 else j
+        elif text.startswith("/*", i):
+            j = text.find("*/", i + 2)
+            i = n if j < 0 else j + 2
+            out.append(" ")
+        else:
+            out.append(c)
+            i += 1
+    return " ".join("".join(out).split())
+
+
 def kernel_sources_digest() -> str:
-    """Digest of the HIP sources the library is built from: a counter run recorded in profiles/ only
-    speaks for the kernels of the same sources."""
+    """Digest of the HIP sources the library is built from, comments and white space left out: a
+    counter run recorded in profiles/ speaks for the kernels of the same code, and an edit of a
+    comment does not change the code."""
     import glob
     import hashlib
     h = hashlib.sha256()
     for path in sorted(glob.glob(os.path.join(ROOT, "adamas_amd", "csrc", "*"))):
-        with open(path, "rb") as f:
-            h.update(os.path.basename(path).encode() + b"\0" + f.read())
+        with open(path, "r", encoding="utf-8") as f:
+            h.update(os.path.basename(path).encode() + b"\0" + strip_c_comments(f.read()).encode())
     return h.hexdigest()[:16]
 
 
@@ -75,15 +102,14 @@ def measured_traffic_bytes(workload: str, kernel: str):
     return int(v) if v is not None else None
 
 
-def estimator_instance(page_size: int, passes: int, chunks: int, heads: int, batch: int,
-                       cus: int) -> str:
-    """Name of the fused estimator's template instance the library launches for these sizes: the
-    heads per workgroup follow the rule of fused_step.hip (narrow workgroups for batches and
-    wherever they leave the busiest CU with fewer bytes)."""
-    wide = chunks * (heads // 8) * batch
-    narrow = batch > 1 or -(-2 * wide // cus) < 2 * -(-wide // cus)
-    return (f"estimate_select_kernel<{16 if page_size == 16 else 0}, {passes}, false, "
-            f"{4 if narrow else 8}>")
+def estimator_instance(_lib, page_size: int, heads: int, batch: int, max_seq_len: int, budget: int) -> str:
+    """Name of the fused estimator's template instance the library launches for these sizes
+    (page size, passes, partial last pass, histogram mode, heads per workgroup, fused projection),
+    from the library's own plan."""
+    p = _lib.step_plan(batch, heads, max_seq_len, budget)
+    flag = lambda v: "true" if v else "false"
+    return (f"estimate_select_kernel<{16 if page_size == 16 else 0}, {p['passes']}, "
+            f"{flag(p['partial'])}, false, {p['heads']}, false>")
 
 
 def log(msg: str) -> None:
@@ -123,6 +149,9 @@ def parse_args():
                          "0.08838834764831845 = 128**-0.5, the orthonormal transform (the library default)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time box of the CPU baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-legs", action="store_true",
+                    help="headline workload only: skip the two extra timings of the step (caches built "
+                         "with the other scale of the transform; a sequence of 33024 tokens)")
     ap.add_argument("--no-e2e", action="store_true",
                     help="skip the end-to-end decode leg (random-init Llama-2-7B shape, 32768-token "
                          "prompt, 256 greedy tokens, sparse path against dense attention)")
@@ -317,8 +346,7 @@ def run_batched(args, w, lib, torch, U, _lib, dev):
         "check": {"against": "estimate + top-k + sparse attention operators, same state",
                   "index_sets": "identical", "max_output_diff": check_err},
         "roofline": {"bound": "hbm",
-                     "kernel": estimator_instance(P, 1, (cap + 511) // 512, H, B,
-                                                  torch.cuda.get_device_properties(dev).multi_processor_count),
+                     "kernel": estimator_instance(_lib, P, H, B, Lmax, budget),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": code_bytes, "avg_launch_us": round(cand_us, 3)},
@@ -380,6 +408,109 @@ def main():
     print(json.dumps(result), flush=True)
 
 
+class StepState:
+    """Resident state of one single-sequence workload: `n_layers` distinct layer caches (token-rolled
+    copies of the same seeded data, shuffled page table), the query codes of the current token and
+    the launch closures of the timed step and of its two kernels."""
+
+    def __init__(self, args, w, L, scale, n_layers, lib, torch, U, _lib, dev, np, synth):
+        import dataclasses
+        H, D, P, budget, Hkv = 32, 128, w.page_size, w.budget, args.kv_heads
+        self.L, self.scale, self.n_layers = L, scale, n_layers
+        seq = synth.make_workload(dataclasses.replace(w, seq_lens=(L,)))[0]
+        self.seq = seq
+        n_pages = (L + P - 1) // P
+        order = np.random.default_rng(w.seed).permutation(n_pages).tolist()   # non-contiguous pages
+        bf16 = args.kv_dtype == "bf16"
+        fdt = torch.bfloat16 if bf16 else torch.float16
+        layout = U.TensorLayout.HND if args.kv_layout == "hnd" else U.TensorLayout.NHD
+        ctrl = U.InferenceController(n_layers, H, D, P, budget, L, fdt, dev, page_order=order,
+                                     num_kv_heads=Hkv, layout=layout, hadamard_scale=scale)
+        self.ctrl, self.fdt = ctrl, fdt
+        kv_flags = ctrl.kv_flags   # the *_f entry points with flags 0 are the plain ones
+        k_dev, v_dev, q_dev = (seq.k[:, :Hkv].to(dev).to(fdt), seq.v[:, :Hkv].to(dev).to(fdt),
+                               seq.q.to(dev).to(fdt))
+        chunk = 8192
+        for s0 in range(0, L - 1, chunk):
+            m = min(chunk, L - 1 - s0)
+            ctrl.prepare_hadamard(m)
+            for layer in range(n_layers):
+                idx = (torch.arange(s0, s0 + m, device=dev) + 997 * layer) % (L - 1)
+                U.append_kvh(k_dev[idx].contiguous(), v_dev[idx].contiguous(), None, ctrl, layer)
+        ctrl.prepare_hadamard(1)
+        ctrl.begin_forward(1)
+        q3 = q_dev[None].contiguous()
+        self.k_new, self.v_new = k_dev[L - 1:].contiguous(), v_dev[L - 1:].contiguous()
+        q_codes = [U.append_kvh(self.k_new, self.v_new, None, ctrl, layer, q=q3)
+                   for layer in range(n_layers)]
+        assert ctrl.need_estimate()
+        torch.cuda.synchronize()
+        self.q3, self.q_codes = q3, q_codes
+        self.ws = ctrl.workspace(budget)
+        self.out = torch.empty_like(q3)
+        self.sel = torch.empty((H, budget - 1), dtype=torch.int32, device=dev)
+        sm_scale = 1.0 / math.sqrt(D)
+        tbl, indptr, lens = (ctrl.seqs.table_dev.data_ptr(), ctrl.seqs.indptr_dev.data_ptr(),
+                             ctrl.seqs.seq_lens_dev.data_ptr())
+        tbl_stride = ctrl.seqs.max_pages   # fixed-stride page tables: rows start at b * max_pages
+        kv_ptr = [ctrl.pool.kv[i].data_ptr() for i in range(n_layers)]
+        code_ptr = [ctrl.pool.codes[i].data_ptr() for i in range(n_layers)]
+        qc_ptr = [c.data_ptr() for c in q_codes]
+        self.ptrs = (tbl, indptr, lens, tbl_stride, kv_ptr, code_ptr, qc_ptr, sm_scale, kv_flags)
+        ws, out, sel = self.ws, self.out, self.sel
+
+        def step(i):
+            ly = i % n_layers
+            rc = lib.adamas_decode_step_f(q3.data_ptr(), qc_ptr[ly], kv_ptr[ly], code_ptr[ly], tbl,
+                                          indptr, lens, budget, out.data_ptr(), sel.data_ptr(),
+                                          ws.data_ptr(), ws.numel(), 1, H, Hkv, D, P, sm_scale, L,
+                                          tbl_stride, kv_flags, _lib.current_stream())
+            if rc:
+                _lib.check(rc, "adamas_decode_step")
+
+        def k_cand(i):
+            ly = i % n_layers
+            rc = lib.adamas_step_candidates(qc_ptr[ly], code_ptr[ly], tbl, indptr, lens, budget,
+                                            ws.data_ptr(), ws.numel(), 1, H, Hkv, P, L, tbl_stride,
+                                            _lib.current_stream())
+            if rc:
+                _lib.check(rc, "adamas_step_candidates")
+
+        def k_attend(i):
+            ly = i % n_layers
+            rc = lib.adamas_step_attend_f(q3.data_ptr(), kv_ptr[ly], code_ptr[ly], tbl, indptr, lens,
+                                          budget, out.data_ptr(), sel.data_ptr(), ws.data_ptr(),
+                                          ws.numel(), 1, H, Hkv, D, P, sm_scale, L, tbl_stride,
+                                          kv_flags, _lib.current_stream())
+            if rc:
+                _lib.check(rc, "adamas_step_attend")
+
+        self.step, self.k_cand, self.k_attend = step, k_cand, k_attend
+
+
+def time_step_leg(args, w, L, scale, lib, torch, U, _lib, dev, np, synth, flush):
+    """The timed step and its two kernels for another sequence length or another scale of the
+    transform than the headline's, same protocol (graph replays behind a cache flush, rotating over
+    the layer caches); the state is released afterwards."""
+    st = StepState(args, w, L, scale, args.layers, lib, torch, U, _lib, dev, np, synth)
+    for i in range(args.warmup):
+        st.step(i)
+    torch.cuda.synchronize()
+    k_iters = (max(64, min(args.steps, 512)) + st.n_layers - 1) // st.n_layers * st.n_layers
+    graph = record_graph(torch, st.step, args.steps)
+    step_us = float(np.median(time_replays(torch, graph, args.steps, 11, flush)))
+    leg = {"value": round(step_us, 3), "unit": "us", "kv_len": L, "hadamard_scale": scale}
+    if lib.adamas_step_fused_supported(1, 32, L, w.budget):
+        leg["estimate_select"] = round(time_graph(torch, st.k_cand, k_iters, flush=flush), 3)
+        st.k_cand(0)
+        leg["select_attend"] = round(time_graph(torch, st.k_attend, k_iters, flush=flush), 3)
+    del graph, st
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    return leg
+
+
 def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
     """The single-sequence kernel workloads (configs 1, 2 and 4): returns the result record."""
     L, budget, P, H, D = w.seq_lens[0], w.budget, w.page_size, 32, 128
@@ -387,59 +518,17 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
     assert H % Hkv == 0
     n_layers = args.layers
     t0 = time.time()
-    seq = synth.make_workload(w)[0]
-    log(f"workload {w.name}: L={L} budget={budget} page={P} generated in {time.time() - t0:.1f}s")
-
-    # ---- build the resident state: n_layers distinct caches (token-rolled copies of the data) ----
-    n_pages = (L + P - 1) // P
-    order = np.random.default_rng(w.seed).permutation(n_pages).tolist()   # non-contiguous pages
-    bf16 = args.kv_dtype == "bf16"
-    fdt = torch.bfloat16 if bf16 else torch.float16
-    layout = U.TensorLayout.HND if args.kv_layout == "hnd" else U.TensorLayout.NHD
-    ctrl = U.InferenceController(n_layers, H, D, P, budget, L, fdt, dev, page_order=order,
-                                 num_kv_heads=Hkv, layout=layout, hadamard_scale=args.hadamard_scale)
-    kv_flags = ctrl.kv_flags   # the *_f entry points with flags 0 are the plain ones
-    k_dev, v_dev, q_dev = (seq.k[:, :Hkv].to(dev).to(fdt), seq.v[:, :Hkv].to(dev).to(fdt),
-                           seq.q.to(dev).to(fdt))
-    chunk = 8192
-    for s0 in range(0, L - 1, chunk):
-        m = min(chunk, L - 1 - s0)
-        ctrl.prepare_hadamard(m)
-        for layer in range(n_layers):
-            idx = (torch.arange(s0, s0 + m, device=dev) + 997 * layer) % (L - 1)
-            U.append_kvh(k_dev[idx].contiguous(), v_dev[idx].contiguous(), None, ctrl, layer)
-    ctrl.prepare_hadamard(1)
-    ctrl.begin_forward(1)
-    q3 = q_dev[None].contiguous()
-    q_codes = [U.append_kvh(k_dev[L - 1:].contiguous(), v_dev[L - 1:].contiguous(), None, ctrl, layer,
-                            q=q3) for layer in range(n_layers)]
-    assert ctrl.need_estimate()
-    torch.cuda.synchronize()
-    log(f"caches resident: {n_layers} layers x ({L * Hkv * D * 4 / 2**20:.0f} MiB KV + "
-        f"{L * Hkv * 32 / 2**20:.0f} MiB codes)")
-
-    ws = ctrl.workspace(budget)
-    out = torch.empty_like(q3)
-    sel = torch.empty((H, budget - 1), dtype=torch.int32, device=dev)
+    st = StepState(args, w, L, args.hadamard_scale, n_layers, lib, torch, U, _lib, dev, np, synth)
+    log(f"workload {w.name}: L={L} budget={budget} page={P}, caches resident after {time.time() - t0:.1f}s: "
+        f"{n_layers} layers x ({L * Hkv * D * 4 / 2**20:.0f} MiB KV + {L * Hkv * 32 / 2**20:.0f} MiB codes)")
+    seq, ctrl, fdt, bf16 = st.seq, st.ctrl, st.fdt, args.kv_dtype == "bf16"
+    q3, ws, out, sel = st.q3, st.ws, st.out, st.sel
+    tbl, indptr, lens, tbl_stride, kv_ptr, code_ptr, qc_ptr, sm_scale, kv_flags = st.ptrs
+    k_new, v_new = st.k_new, st.v_new
+    step, k_cand, k_attend = st.step, st.k_cand, st.k_attend
     dist = torch.empty((H, (L + 7) // 8 * 8), dtype=torch.int16, device=dev)
     topk_ws = torch.zeros(lib.adamas_topk_workspace_bytes(H, L - 1, budget - 1), dtype=torch.uint8,
                           device=dev)
-    sm_scale = 1.0 / math.sqrt(D)
-    tbl, indptr, lens = (ctrl.seqs.table_dev.data_ptr(), ctrl.seqs.indptr_dev.data_ptr(),
-                         ctrl.seqs.seq_lens_dev.data_ptr())
-    tbl_stride = ctrl.seqs.max_pages   # fixed-stride page tables: rows start at b * max_pages
-    kv_ptr = [ctrl.pool.kv[i].data_ptr() for i in range(n_layers)]
-    code_ptr = [ctrl.pool.codes[i].data_ptr() for i in range(n_layers)]
-    qc_ptr = [c.data_ptr() for c in q_codes]
-
-    def step(i):
-        ly = i % n_layers
-        rc = lib.adamas_decode_step_f(q3.data_ptr(), qc_ptr[ly], kv_ptr[ly], code_ptr[ly], tbl,
-                                      indptr, lens, budget, out.data_ptr(), sel.data_ptr(),
-                                      ws.data_ptr(), ws.numel(), 1, H, Hkv, D, P, sm_scale, L,
-                                      tbl_stride, kv_flags, _lib.current_stream())
-        if rc:
-            _lib.check(rc, "adamas_decode_step")
 
     def k_estimate(i):
         ly = i % n_layers
@@ -473,25 +562,7 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         if rc:
             _lib.check(rc, "adamas_sparse_decode (dense)")
 
-    def k_cand(i):
-        ly = i % n_layers
-        rc = lib.adamas_step_candidates(qc_ptr[ly], code_ptr[ly], tbl, indptr, lens, budget,
-                                        ws.data_ptr(), ws.numel(), 1, H, Hkv, P, L, tbl_stride,
-                                        _lib.current_stream())
-        if rc:
-            _lib.check(rc, "adamas_step_candidates")
-
-    def k_attend(i):
-        ly = i % n_layers
-        rc = lib.adamas_step_attend_f(q3.data_ptr(), kv_ptr[ly], code_ptr[ly], tbl, indptr, lens,
-                                      budget, out.data_ptr(), sel.data_ptr(), ws.data_ptr(),
-                                      ws.numel(), 1, H, Hkv, D, P, sm_scale, L, tbl_stride, kv_flags,
-                                      _lib.current_stream())
-        if rc:
-            _lib.check(rc, "adamas_step_attend")
-
     dense_flags = kv_flags | (_lib.F_NO_MFMA if args.gqa_vector_alu else 0)
-    k_new, v_new = k_dev[L - 1:].contiguous(), v_dev[L - 1:].contiguous()
     qc_tmp = torch.empty((1, H, 16), dtype=torch.int16, device=dev)
 
     def k_append(i):
@@ -594,13 +665,27 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
     check_err = check_against_operators(np, out_step, sel_step, out, sel, w.name)
     log(f"timed step == stand-alone operators (identical index sets, max output difference {check_err:.1e})")
 
+    # ---- the same step on the other scale of the transform and just past the headline length ------
+    # (the headline workload only: caches built with the orthonormal transform, whose codes take two
+    # of the four levels on these inputs, and a sequence of 33024 tokens, which is what a decode loop
+    # sees a few hundred tokens after a 32768-token prompt)
+    extra_legs = {}
+    if (args.workload == "c2_32k_b128" and (L, budget) == (32768, 128) and Hkv == H and not bf16
+            and args.kv_layout == "nhd" and not args.no_extra_legs):
+        other = U.ORTHONORMAL_SCALE if args.hadamard_scale == 1.0 else 1.0
+        key = "orthonormal_scale" if other == U.ORTHONORMAL_SCALE else "raw_scale"
+        extra_legs[key] = time_step_leg(args, w, L, other, lib, torch, U, _lib, dev, np, synth, flush)
+        extra_legs["kv_len_33024"] = time_step_leg(args, w, 33024, args.hadamard_scale, lib, torch, U,
+                                                   _lib, dev, np, synth, flush)
+        for name, leg in extra_legs.items():
+            log(f"{name}: step {leg['value']:.2f} us (estimate+select {leg.get('estimate_select')}, "
+                f"select+attend {leg.get('select_attend')})")
+
     # ---- roofline of the dominant kernel of the timed step: the fused estimator -----------------
     # algorithmic bytes of one launch = the 2-bit codes of the L-1 past tokens (32 bytes per token
     # and head); what the kernel writes (candidates, histograms) is overhead, not counted
-    passes = next((p for p in (1, 2, 4) if -(-(L - 1) // (512 * p)) * ((budget + 6) // 8 * 8) <= 16384), 4)
-    dom_name, dom_us = ((estimator_instance(P, passes, -(-(L - 1) // (512 * passes)), H, 1,
-                                            torch.cuda.get_device_properties(dev).multi_processor_count),
-                         cand_us) if fused else (f"estimate_kernel<{16 if P == 16 else 0}>", est_us))
+    dom_name, dom_us = ((estimator_instance(_lib, P, H, 1, L, budget), cand_us) if fused
+                        else (f"estimate_kernel<{16 if P == 16 else 0}>", est_us))
     est_bytes = (L - 1) * Hkv * 32
     step_bytes = L * Hkv * (D // 4) + 2 * budget * H * D * 2   # codes + selected K and V rows
     achieved = est_bytes / (dom_us * 1e-6) / 1e9
@@ -686,6 +771,7 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
+    result.update(extra_legs)
     return result
 
 

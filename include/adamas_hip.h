@@ -311,6 +311,15 @@ int adamas_decode_step_noalloc(const void* q, const void* q_code, const void* kv
  */
 int adamas_step_fused_supported(uint32_t batch, uint32_t num_heads, uint32_t max_seq_len,
                                 uint32_t budget);
+/*
+ * How the two-launch step cuts these sizes up (host arithmetic only, for tools and tests; no
+ * counterpart in the reference).  plan_out receives 8 values: supported (0/1), heads per workgroup of
+ * the first launch (8 or 4), chunks per sequence, 16-token units per chunk (quotient), chunks that
+ * have one unit more (remainder), passes of 512 tokens per workgroup, whether the last pass can be
+ * partial (0/1), candidate slots per head and chunk.
+ */
+int adamas_step_plan(uint32_t batch, uint32_t num_heads, uint32_t max_seq_len, uint32_t budget,
+                     uint32_t* plan_out);
 int adamas_step_candidates(const void* q_code, const void* code_data, const int32_t* page_indices,
                            const int32_t* page_indptr, const int32_t* seq_lens, uint32_t budget,
                            void* workspace, size_t workspace_bytes, uint32_t batch,
