@@ -59,8 +59,9 @@ struct EstimateSelectShared {
 };
 
 // Where the query comes from when a kernel of the step takes the fused q/k/v projection of the
-// decoder instead of a rotated query and its code: qkv [batch][Hq + 2*Hkv][128] fp16, rotary tables
-// [positions][64] fp32 (rotate-half pairing), and the parameters of the code generation.
+// decoder instead of a rotated query and its code: qkv [batch][Hq + 2*Hkv][128] fp16 or bf16
+// (ADAMAS_F_BF16 in code_flags), rotary tables [positions][64] fp32 (rotate-half pairing), and the
+// parameters of the code generation.
 struct QkvSource {
   const __half* qkv = nullptr;
   const float* cos_table = nullptr;
@@ -100,15 +101,33 @@ __device__ __forceinline__ WaveRopeLoads wave_rope_load(const __half* row, const
   return r;
 }
 
-// x0, x1: the rotated channels rounded to fp16, as a stored tensor would hold them
+// x0, x1: the rotated channels rounded to the 16-bit format, as a stored tensor would hold them
+template <bool kBf16>
 __device__ __forceinline__ void wave_rope_apply(const WaveRopeLoads& r, int lane, float& x0,
                                                 float& x1) {
   float q0, q1;
-  unpack2<false>(r.raw, q0, q1);
+  unpack2<kBf16>(r.raw, q0, q1);
   const bool upper = lane >= 32;  // channels 64 .. 127 pair with the lane 32 below
   const float p0 = __shfl_xor(q0, 32), p1 = __shfl_xor(q1, 32);
-  x0 = round_elem<false>(rope_channel(q0, p0, r.cs.x, r.sn.x, upper));
-  x1 = round_elem<false>(rope_channel(q1, p1, r.cs.y, r.sn.y, upper));
+  x0 = round_elem<kBf16>(rope_channel(q0, p0, r.cs.x, r.sn.x, upper));
+  x1 = round_elem<kBf16>(rope_channel(q1, p1, r.cs.y, r.sn.y, upper));
+}
+
+// The query code of a row of the fused projection (rotary embedding, transform, buckets) with the
+// format known at run time only (uniform over the launch): the estimator is not instantiated twice
+// for something a wave does once.
+__device__ __forceinline__ uint32_t wave_query_code(const WaveRopeLoads& r, int lane, float scale,
+                                                    uint32_t code_flags) {
+  float x0, x1;
+  const bool keep = (code_flags & ADAMAS_F_CODE_FROM_FP32) != 0;
+  if (code_flags & ADAMAS_F_BF16) {
+    wave_rope_apply<true>(r, lane, x0, x1);
+    transform_row<true>(x0, x1, lane, scale, keep);
+  } else {
+    wave_rope_apply<false>(r, lane, x0, x1);
+    transform_row<false>(x0, x1, lane, scale, keep);
+  }
+  return wave_pack_codes(x0, x1, lane);
 }
 
 // kPartial: chunks may be shorter than kPasses * 512 tokens by whole 16-token units (balanced chunks
@@ -305,10 +324,7 @@ __global__ __launch_bounds__(kHeads * kWave) void estimate_select_kernel(
       *reinterpret_cast<uint4*>(qcode_out + (static_cast<size_t>(b) * num_heads + head) * kCodeWords +
                                 half * 8u) = qraw_copy;
     if (kFromQkv) {
-      float qx0, qx1;
-      wave_rope_apply(qload, lane, qx0, qx1);
-      transform_row(qx0, qx1, lane, src.scale, (src.code_flags & ADAMAS_F_CODE_FROM_FP32) != 0);
-      const uint32_t word = wave_pack_codes(qx0, qx1, lane);
+      const uint32_t word = wave_query_code(qload, lane, src.scale, src.code_flags);
       if ((lane & 3) == 0) {
         sh.qcode[wave][lane >> 2] = static_cast<uint16_t>(word);
         if (chunk == 0)
@@ -417,11 +433,10 @@ struct SelectAttendShared {
 // q_code [sequence*heads][16], code_data: the query codes and the code cache the first launch worked
 // with, read only when a chunk has to be scored again; dist_scratch [sequence*heads][dist_stride]
 // u16 then holds that chunk's distances (rows are private to a workgroup).
-// kFromQkv (fp16, NHD pages): q is not read; the kernel takes the fused projection of the decoder,
-// applies the rotary embedding to the query and to the new key itself, appends the new key, its code
-// and the new value (the workgroup of the first query head of a key/value head), and attends the
-// current token from registers instead of reading it back: the decode append needs no launch of its
-// own.
+// kFromQkv: q is not read; the kernel takes the fused projection of the decoder, applies the rotary
+// embedding to the query and to the new key itself, appends the new key, its code and the new value
+// (the workgroup of the first query head of a key/value head), and attends the current token from
+// registers instead of reading it back: the decode append needs no launch of its own.
 template <bool kBf16, bool kHnd, bool kFromQkv = false>
 __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     const __half* __restrict__ q, const __half* __restrict__ kv_data,
@@ -433,7 +448,6 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     const uint16_t* __restrict__ q_code, const unsigned char* code_data,
     uint16_t* __restrict__ dist_scratch, int64_t dist_stride, QkvSource src = QkvSource(),
     __half* kv_append = nullptr, uint16_t* code_append = nullptr) {
-  static_assert(!kFromQkv || (!kBf16 && !kHnd), "the fused projection is fp16 over NHD pages");
   static_assert(kAttThreads == kHistBins, "one thread per distance value");
   static_assert(kStepMaxSlots == 2 * kAttThreads, "two candidate slots per thread");
   static_assert(kStepMaxChunks == kWave, "the flags of all chunks fit one ballot");
@@ -518,15 +532,15 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   if (kFromQkv && wave < 3) {
     float x0, x1;
     if (wave == 2) {  // the value row is taken as it is
-      unpack2<false>(row_now.raw, x0, x1);
+      unpack2<kBf16>(row_now.raw, x0, x1);
     } else {
-      wave_rope_apply(row_now, lane, x0, x1);
+      wave_rope_apply<kBf16>(row_now, lane, x0, x1);
     }
     const float f = wave == 0 ? scale_log2 : 1.0f;
     *reinterpret_cast<float2*>(&sh.qkv_now[wave][2 * lane]) = make_float2(x0 * f, x1 * f);
     if (wave == 1) {
-      kpacked = pack2<false>(x0, x1);
-      transform_row(x0, x1, lane, src.scale, (src.code_flags & ADAMAS_F_CODE_FROM_FP32) != 0);
+      kpacked = pack2<kBf16>(x0, x1);
+      transform_row<kBf16>(x0, x1, lane, src.scale, (src.code_flags & ADAMAS_F_CODE_FROM_FP32) != 0);
       kcode_word = wave_pack_codes(x0, x1, lane);
     }
   }
@@ -713,17 +727,17 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     if (appends && (wave == 1 || wave == 2)) {
       // the new token goes into the caches after every read of them: wave 1 writes K (rotated) and
       // its code, wave 2 writes V
-      const size_t tok_stride = static_cast<size_t>(num_kv_heads) * kHeadDim;
-      __half* krow_p = kv_append +
-                       (static_cast<size_t>(cur_page) * 2 * page_size + cur_slot) * tok_stride +
-                       static_cast<size_t>(kv_head_now) * kHeadDim;
+      const uint32_t lay = kHnd ? ADAMAS_F_HND : 0u;
       if (wave == 1) {
-        reinterpret_cast<uint32_t*>(krow_p)[lane] = kpacked;
+        reinterpret_cast<uint32_t*>(kv_append + kv_row_offset(cur_page, 0, cur_slot, kv_head_now,
+                                                              page_size, num_kv_heads, lay))[lane] =
+            kpacked;
         if ((lane & 3) == 0)
           code_append[((static_cast<size_t>(cur_page) * page_size + cur_slot) * num_kv_heads +
                        kv_head_now) * kCodeWords + (lane >> 2)] = static_cast<uint16_t>(kcode_word);
       } else {
-        reinterpret_cast<uint32_t*>(krow_p + static_cast<size_t>(page_size) * tok_stride)[lane] =
+        reinterpret_cast<uint32_t*>(kv_append + kv_row_offset(cur_page, 1, cur_slot, kv_head_now,
+                                                              page_size, num_kv_heads, lay))[lane] =
             row_now.raw;
       }
     }
@@ -926,10 +940,7 @@ static int step_attend_impl(const void* q, void* kv_data, void* code_data,
                             uint32_t max_seq_len, uint32_t page_table_stride, uint32_t flags,
                             adamas_stream_t stream, const QkvSource* qsrc) {
   if (flags & ~(ADAMAS_F_BF16 | ADAMAS_F_HND)) return ADAMAS_E_BADARG;
-  if (qsrc) {
-    if (flags != 0) return ADAMAS_E_UNSUPPORTED;
-    q = qsrc->qkv;
-  }
+  if (qsrc) q = qsrc->qkv;
   const bool bf16 = (flags & ADAMAS_F_BF16) != 0;
   const bool hnd = (flags & ADAMAS_F_HND) != 0;
   if (!q || !kv_data || !code_data || !page_indices || (!page_indptr && !page_table_stride) ||
@@ -965,17 +976,22 @@ static int step_attend_impl(const void* q, void* kv_data, void* code_data,
                      reinterpret_cast<uint16_t*>(ws + w.dist_off), w.dist_stride,               \
                      qsrc ? *qsrc : QkvSource(), static_cast<__half*>(kv_data),                 \
                      static_cast<uint16_t*>(code_data))
-  if (qsrc) {
-    ADAMAS_LAUNCH_SELATT_BF(false, false, true);
-  } else if (bf16 && hnd) {
-    ADAMAS_LAUNCH_SELATT_BF(true, true, false);
-  } else if (bf16) {
-    ADAMAS_LAUNCH_SELATT_BF(true, false, false);
-  } else if (hnd) {
-    ADAMAS_LAUNCH_SELATT_BF(false, true, false);
-  } else {
-    ADAMAS_LAUNCH_SELATT_BF(false, false, false);
+#define ADAMAS_LAUNCH_SELATT(FROMQKV)                 \
+  if (bf16 && hnd) {                                  \
+    ADAMAS_LAUNCH_SELATT_BF(true, true, FROMQKV);     \
+  } else if (bf16) {                                  \
+    ADAMAS_LAUNCH_SELATT_BF(true, false, FROMQKV);    \
+  } else if (hnd) {                                   \
+    ADAMAS_LAUNCH_SELATT_BF(false, true, FROMQKV);    \
+  } else {                                            \
+    ADAMAS_LAUNCH_SELATT_BF(false, false, FROMQKV);   \
   }
+  if (qsrc) {
+    ADAMAS_LAUNCH_SELATT(true)
+  } else {
+    ADAMAS_LAUNCH_SELATT(false)
+  }
+#undef ADAMAS_LAUNCH_SELATT
 #undef ADAMAS_LAUNCH_SELATT_BF
   ADAMAS_RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -1151,7 +1167,7 @@ extern "C" int adamas_decode_layer_step(const void* qkv, const float* cos_table,
                                         float hadamard_scale, uint32_t flags,
                                         adamas_stream_t stream) {
   if (!qkv || !cos_table || !sin_table || !kv_data || !code_data) return ADAMAS_E_BADARG;
-  if (flags & ~ADAMAS_F_CODE_FROM_FP32) return ADAMAS_E_UNSUPPORTED;  // fp16, NHD pages only
+  if (flags & ~(ADAMAS_F_CODE_FROM_FP32 | ADAMAS_F_BF16 | ADAMAS_F_HND)) return ADAMAS_E_BADARG;
   if ((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(cos_table) |
        reinterpret_cast<uintptr_t>(sin_table)) & 15)
     return ADAMAS_E_ALIGN;
@@ -1161,14 +1177,15 @@ extern "C" int adamas_decode_layer_step(const void* qkv, const float* cos_table,
   src.sin_table = sin_table;
   src.scale = hadamard_scale;
   src.code_flags = flags;
+  const uint32_t kv_flags = flags & (ADAMAS_F_BF16 | ADAMAS_F_HND);  // format and layout of the caches
   int rc = step_candidates_impl(nullptr, code_data, page_indices, page_indptr, seq_lens, budget,
                                 workspace, workspace_bytes, batch, num_heads, num_kv_heads,
-                                page_size, max_seq_len, page_table_stride, 0u, stream, &src);
+                                page_size, max_seq_len, page_table_stride, kv_flags, stream, &src);
   if (rc != 0) return rc;
   return step_attend_impl(nullptr, kv_data, code_data, page_indices, page_indptr, seq_lens, budget,
                           out, sel_out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
-                          head_dim, page_size, sm_scale, max_seq_len, page_table_stride, 0u, stream,
-                          &src);
+                          head_dim, page_size, sm_scale, max_seq_len, page_table_stride, kv_flags,
+                          stream, &src);
 }
 
 // ---- the decode step for callers that cannot allocate ----------------------------------------------

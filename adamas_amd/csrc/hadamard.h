@@ -126,6 +126,15 @@ __device__ __forceinline__ void unpack_elem8(const uint4& raw, float (&x)[8]) {
 }
 
 
+// element offset of the K (kv = 0) or V (kv = 1) row of (page, slot, head) in a KV page pool:
+// pages are [2][page_size][heads][128], or [2][heads][page_size][128] with ADAMAS_F_HND
+__device__ __forceinline__ size_t kv_row_offset(size_t page, uint32_t kv, uint32_t slot, uint32_t hd,
+                                                uint32_t page_size, uint32_t num_heads,
+                                                uint32_t flags) {
+  if (flags & ADAMAS_F_HND) return (((page * 2 + kv) * num_heads + hd) * page_size + slot) * kHeadDim;
+  return (((page * 2 + kv) * page_size + slot) * num_heads + hd) * kHeadDim;
+}
+
 // Rotary embedding of one channel pair (c, c + 64) in rotate-half pairing: `x` is this lane's
 // value, `partner` the value of the paired channel, `upper` whether this lane holds the channel
 // c + 64.  lower: x*cos - partner*sin, upper: x*cos + partner*sin; two products and one sum, each

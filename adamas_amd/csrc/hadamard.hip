@@ -55,15 +55,6 @@ __global__ __launch_bounds__(256) void pack_2bit_kernel(const __half* __restrict
   }
 }
 
-// element offset of the K (kv = 0) or V (kv = 1) row of (page, slot, head) in a KV page pool:
-// pages are [2][page_size][heads][128], or [2][heads][page_size][128] with ADAMAS_F_HND
-__device__ __forceinline__ size_t kv_row_offset(size_t page, uint32_t kv, uint32_t slot, uint32_t hd,
-                                                uint32_t page_size, uint32_t num_heads,
-                                                uint32_t flags) {
-  if (flags & ADAMAS_F_HND) return (((page * 2 + kv) * num_heads + hd) * page_size + slot) * kHeadDim;
-  return (((page * 2 + kv) * page_size + slot) * num_heads + hd) * kHeadDim;
-}
-
 // ------------------------------------------------------------------------------------------------
 // Decode append: rows [0, batch*Hq) are query rows, rows [batch*Hq, batch*(Hq+Hkv)) are key rows.
 // ------------------------------------------------------------------------------------------------
@@ -124,6 +115,7 @@ __global__ __launch_bounds__(256) void append_decode_kernel(
 // Hadamard(q) and Hadamard(k) to q_code_out and the code page.  The rotated values are rounded to fp16
 // before the transform, exactly as if they had been stored and appended separately.
 // ------------------------------------------------------------------------------------------------
+template <bool kBf16>
 __global__ __launch_bounds__(256) void rope_append_decode_kernel(
     const __half* __restrict__ qkv, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, __half* __restrict__ q_out,
@@ -144,8 +136,8 @@ __global__ __launch_bounds__(256) void rope_append_decode_kernel(
   const size_t row_len = static_cast<size_t>(num_q_heads + 2 * num_heads) * kHeadDim;
   const __half* row = qkv + static_cast<size_t>(b) * row_len;
   float q0, q1, k0 = 0.f, k1 = 0.f;
-  load_pair(row + static_cast<size_t>(hd) * kHeadDim, lane, q0, q1);
-  if (has_kv) load_pair(row + static_cast<size_t>(num_q_heads + hd) * kHeadDim, lane, k0, k1);
+  load_pair<kBf16>(row + static_cast<size_t>(hd) * kHeadDim, lane, q0, q1);
+  if (has_kv) load_pair<kBf16>(row + static_cast<size_t>(num_q_heads + hd) * kHeadDim, lane, k0, k1);
 
   // channel c pairs with c + 64 (lanes l and l + 32): out_lo = lo*cos - hi*sin, out_hi = hi*cos + lo*sin
   const uint32_t c0 = (2u * static_cast<uint32_t>(lane)) & 63u;  // table column of channel 2l
@@ -154,15 +146,15 @@ __global__ __launch_bounds__(256) void rope_append_decode_kernel(
   const bool upper = lane >= 32;
   const float pq0 = __shfl_xor(q0, 32), pq1 = __shfl_xor(q1, 32);
   const float pk0 = __shfl_xor(k0, 32), pk1 = __shfl_xor(k1, 32);
-  const __half2 qh = __floats2half2_rn(upper ? q0 * cs.x + pq0 * sn.x : q0 * cs.x - pq0 * sn.x,
-                                       upper ? q1 * cs.y + pq1 * sn.y : q1 * cs.y - pq1 * sn.y);
-  const __half2 kh = __floats2half2_rn(upper ? k0 * cs.x + pk0 * sn.x : k0 * cs.x - pk0 * sn.x,
-                                       upper ? k1 * cs.y + pk1 * sn.y : k1 * cs.y - pk1 * sn.y);
-  reinterpret_cast<__half2*>(q_out + static_cast<size_t>(bh) * kHeadDim)[lane] = qh;
+  // the rotated values as a stored tensor of the data's format holds them
+  float x0 = round_elem<kBf16>(rope_channel(q0, pq0, cs.x, sn.x, upper));
+  float x1 = round_elem<kBf16>(rope_channel(q1, pq1, cs.y, sn.y, upper));
+  const float kr0 = round_elem<kBf16>(rope_channel(k0, pk0, cs.x, sn.x, upper));
+  const float kr1 = round_elem<kBf16>(rope_channel(k1, pk1, cs.y, sn.y, upper));
+  reinterpret_cast<uint32_t*>(q_out + static_cast<size_t>(bh) * kHeadDim)[lane] = pack2<kBf16>(x0, x1);
 
   const bool keep_fp32 = (flags & ADAMAS_F_CODE_FROM_FP32) != 0;
-  float x0 = __low2float(qh), x1 = __high2float(qh);
-  transform_row(x0, x1, lane, scale, keep_fp32);
+  transform_row<kBf16>(x0, x1, lane, scale, keep_fp32);
   const uint32_t qword = wave_pack_codes(x0, x1, lane);
   if ((lane & 3) == 0)
     q_code_out[static_cast<size_t>(bh) * kCodeWords + (lane >> 2)] = static_cast<uint16_t>(qword);
@@ -174,13 +166,13 @@ __global__ __launch_bounds__(256) void rope_append_decode_kernel(
   const size_t page = static_cast<size_t>(table[lp]);
   const uint32_t vraw =
       reinterpret_cast<const uint32_t*>(row + static_cast<size_t>(num_q_heads + num_heads + hd) * kHeadDim)[lane];
-  const size_t k_off = (((page * 2 + 0) * page_size + slot) * num_heads + hd) * kHeadDim;
-  const size_t v_off = (((page * 2 + 1) * page_size + slot) * num_heads + hd) * kHeadDim;
-  reinterpret_cast<__half2*>(kv_data + k_off)[lane] = kh;
+  const size_t k_off = kv_row_offset(page, 0, slot, hd, page_size, num_heads, flags);
+  const size_t v_off = kv_row_offset(page, 1, slot, hd, page_size, num_heads, flags);
+  reinterpret_cast<uint32_t*>(kv_data + k_off)[lane] = pack2<kBf16>(kr0, kr1);
   reinterpret_cast<uint32_t*>(kv_data + v_off)[lane] = vraw;
-  x0 = __low2float(kh);
-  x1 = __high2float(kh);
-  transform_row(x0, x1, lane, scale, keep_fp32);
+  x0 = kr0;
+  x1 = kr1;
+  transform_row<kBf16>(x0, x1, lane, scale, keep_fp32);
   const uint32_t kword = wave_pack_codes(x0, x1, lane);
   if ((lane & 3) == 0)
     code_data[((page * page_size + slot) * num_heads + hd) * kCodeWords + (lane >> 2)] =
@@ -354,16 +346,20 @@ extern "C" int adamas_rope_append_decode(const void* qkv, const float* cos_table
       num_kv_heads == 0 || page_size == 0)
     return ADAMAS_E_BADARG;
   if (head_dim != kHeadDim || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
-  // the decoder operators are fp16 / NHD only
-  if (flags & (ADAMAS_F_BF16 | ADAMAS_F_HND)) return ADAMAS_E_UNSUPPORTED;
+  if (flags & ~(ADAMAS_F_BF16 | ADAMAS_F_HND | ADAMAS_F_CODE_FROM_FP32)) return ADAMAS_E_BADARG;
   if ((reinterpret_cast<uintptr_t>(cos_table) | reinterpret_cast<uintptr_t>(sin_table)) & 7)
     return ADAMAS_E_ALIGN;
   const uint32_t rows = batch * num_heads;
-  hipLaunchKernelGGL(rope_append_decode_kernel, dim3((rows + 3) / 4), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const __half*>(qkv), cos_table,
-                     sin_table, static_cast<__half*>(q_out), static_cast<uint16_t*>(q_code_out),
-                     static_cast<__half*>(kv_data), static_cast<uint16_t*>(code_data), page_indices,
-                     page_indptr, seq_lens, batch, num_heads, num_kv_heads, page_size, scale, flags);
+#define ADAMAS_LAUNCH_ROPE_APPEND(BF)                                                              \
+  hipLaunchKernelGGL(rope_append_decode_kernel<BF>, dim3((rows + 3) / 4), dim3(256), 0,            \
+                     static_cast<hipStream_t>(stream), static_cast<const __half*>(qkv), cos_table, \
+                     sin_table, static_cast<__half*>(q_out), static_cast<uint16_t*>(q_code_out),   \
+                     static_cast<__half*>(kv_data), static_cast<uint16_t*>(code_data),             \
+                     page_indices, page_indptr, seq_lens, batch, num_heads, num_kv_heads,          \
+                     page_size, scale, flags)
+  if (flags & ADAMAS_F_BF16) ADAMAS_LAUNCH_ROPE_APPEND(true);
+  else ADAMAS_LAUNCH_ROPE_APPEND(false);
+#undef ADAMAS_LAUNCH_ROPE_APPEND
   ADAMAS_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

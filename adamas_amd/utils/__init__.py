@@ -616,7 +616,7 @@ def rope_append_decode(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: to
     rotated, q_code [B, Hq, 16]): the same tensors rope_split followed by
     append_kvh(k, v, None, ..., q=q) produce (Adamas.py:113 and :145-155 in the reference)."""
     c = iController
-    _check_cuda_contig(qkv, "qkv", torch.float16)
+    _check_cuda_contig(qkv, "qkv", c.dtype)
     _check_cuda_contig(cos_table, "cos_table", torch.float32, 2)
     _check_cuda_contig(sin_table, "sin_table", torch.float32, 2)
     n, nq, nkv = _qkv_heads(qkv, c.num_kv_heads)
@@ -626,7 +626,7 @@ def rope_append_decode(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: to
         raise RuntimeError("rotary tables must be [positions >= sequence length, 64]")
     if c.min_len_now < 1:
         raise RuntimeError("prepare_hadamard must reserve the token before the append")
-    q = torch.empty((n, nq, 128), dtype=torch.float16, device=qkv.device)
+    q = torch.empty((n, nq, 128), dtype=c.dtype, device=qkv.device)
     q_code = torch.empty((n, nq, 16), dtype=torch.int16, device=qkv.device)
     rc = _lib.load().adamas_rope_append_decode(
         qkv.data_ptr(), cos_table.data_ptr(), sin_table.data_ptr(), q.data_ptr(), q_code.data_ptr(),
@@ -690,10 +690,10 @@ def sumsq_partials(x: torch.Tensor, partials: torch.Tensor) -> None:
 
 
 def layer_step_supported(iController: InferenceController) -> bool:
-    """Whether decode_layer_step serves the controller's current sizes (fp16, NHD pages, a budget and
-    lengths the two-launch step covers); otherwise use rope_append_decode + decode_step."""
+    """Whether decode_layer_step serves the controller's current sizes (a budget and lengths the
+    two-launch step covers); otherwise use rope_append_decode + decode_step."""
     c = iController
-    if c.dtype != torch.float16 or c.layout != TensorLayout.NHD or c.inference_page_budget is None:
+    if c.inference_page_budget is None:
         return False
     return bool(_lib.load().adamas_step_fused_supported(c.batch_size, c.num_heads, c.max_len_now,
                                                         c.inference_page_budget))
@@ -708,9 +708,7 @@ def decode_layer_step(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: tor
     o [B, Hq, 128] and, on request, the selected positions.  The controller must have reserved the
     token (prepare_hadamard / begin_forward, or a graph decode)."""
     c = iController
-    if c.dtype != torch.float16 or c.layout != TensorLayout.NHD:
-        raise RuntimeError("decode_layer_step serves float16 caches with NHD pages only")
-    _check_cuda_contig(qkv, "qkv", torch.float16)
+    _check_cuda_contig(qkv, "qkv", c.dtype)
     _check_cuda_contig(cos_table, "cos_table", torch.float32, 2)
     _check_cuda_contig(sin_table, "sin_table", torch.float32, 2)
     nq, nkv = c.num_heads, c.num_kv_heads
@@ -724,7 +722,7 @@ def decode_layer_step(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: tor
     if c.min_len_now < 1:
         raise RuntimeError("prepare_hadamard must reserve the token before the step")
     budget = c.inference_page_budget
-    o = torch.empty((n, nq, 128), dtype=torch.float16, device=qkv.device)
+    o = torch.empty((n, nq, 128), dtype=c.dtype, device=qkv.device)
     ws = c.workspace(budget)
     sel = c.topk_dindices_buffer if return_indices else None
     rc = _lib.load().adamas_decode_layer_step(
@@ -732,7 +730,7 @@ def decode_layer_step(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: tor
         c.pool.codes[layer_idx].data_ptr(), c.seqs.table_dev.data_ptr(), c.seqs.indptr_dev.data_ptr(),
         c.seqs.seq_lens_dev.data_ptr(), budget, o.data_ptr(), _lib.ptr(sel), ws.data_ptr(), ws.numel(),
         n, nq, nkv, 128, c.page_size, 1.0 / math.sqrt(c.head_dim), c.max_len_now, c.seqs.max_pages,
-        c.hadamard_scale, c.code_flags & _lib.F_CODE_FROM_FP32, _lib.current_stream())
+        c.hadamard_scale, c.code_flags, _lib.current_stream())
     _lib.check(rc, "adamas_decode_layer_step")
     return (o, sel) if return_indices else o
 

@@ -389,6 +389,8 @@ int adamas_rope_in_place(void* q, void* k, uint32_t rows, uint32_t num_heads, ui
  * [batch][num_heads][128], rotated k and v into the KV page, the codes of Hadamard(q) to q_code_out
  * and of Hadamard(k) into the code page.  Same results as adamas_rope_split followed by
  * adamas_append_decode (adamas/models/Adamas.py:113 and :145-155 in the reference), one launch.
+ * flags: ADAMAS_F_BF16 (qkv, q_out and the KV pages hold bfloat16), ADAMAS_F_HND (page layout),
+ * ADAMAS_F_CODE_FROM_FP32.
  */
 int adamas_rope_append_decode(const void* qkv, const float* cos_table, const float* sin_table,
                               void* q_out, void* q_code_out, void* kv_data, void* code_data,
@@ -407,8 +409,9 @@ int adamas_rope_append_decode(const void* qkv, const float* cos_table, const flo
  * into the caches and attends the selected tokens plus the new one (from registers).  Results are
  * those of the two-call sequence: identical codes, cache contents and selections, outputs equal up
  * to the order of the softmax accumulation.
- * fp16 and NHD pages only; flags: ADAMAS_F_CODE_FROM_FP32.  Returns ADAMAS_E_UNSUPPORTED where
- * adamas_step_fused_supported() is 0 (the caller then uses the two-call sequence).
+ * flags: ADAMAS_F_BF16 (qkv, the KV pages and out hold bfloat16), ADAMAS_F_HND (page layout),
+ * ADAMAS_F_CODE_FROM_FP32.  Returns ADAMAS_E_UNSUPPORTED where adamas_step_fused_supported() is 0
+ * (the caller then uses the two-call sequence).
  * No counterpart in the reference (its decode step is apply_rope_in_place, append_kv_cache_decode,
  * estimate, top-k and attention as separate launches, adamas/models/Adamas.py:129-201).
  */

@@ -267,12 +267,16 @@ def test_rope_append_decode_equals_rope_split_plus_append(gpu_device):
     ([9000], 32, 32, 1, 200),            # page size 1
 ])
 @pytest.mark.parametrize("scale", [1.0, 128 ** -0.5])
-def test_layer_step_equals_append_then_step(gpu_device, lens, hq, hkv, page_size, budget, scale):
+@pytest.mark.parametrize("fmt", ["fp16-nhd", "bf16-nhd", "fp16-hnd", "bf16-hnd"])
+def test_layer_step_equals_append_then_step(gpu_device, lens, hq, hkv, page_size, budget, scale, fmt):
     """adamas_decode_layer_step (query code, rotary embedding, append and step in two launches)
     against rope_append_decode + decode_step: same cache contents and codes bit for bit, same
-    selections, outputs equal up to the order of the softmax accumulation."""
+    selections, outputs equal up to the order of the softmax accumulation; float16 and bfloat16
+    data, both page layouts."""
     import adamas_amd.utils as U
     from tests import helpers as T
+    dtype = torch.bfloat16 if fmt.startswith("bf16") else torch.float16
+    layout = U.TensorLayout.HND if fmt.endswith("hnd") else U.TensorLayout.NHD
     B, D = len(lens), 128
     cap = max(lens) + 8
     g = torch.Generator().manual_seed(sum(lens) + hq)
@@ -280,13 +284,14 @@ def test_layer_step_equals_append_then_step(gpu_device, lens, hq, hkv, page_size
     inv = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) / half))
     ang = torch.arange(cap, dtype=torch.float64)[:, None] * inv[None, :]
     cos, sin = ang.cos().float().to(gpu_device), ang.sin().float().to(gpu_device)
-    qkv = (torch.randn(B, hq + 2 * hkv, D, generator=g) * 2).half().to(gpu_device)
-    past = [((torch.randn(L - 1, hkv, D, generator=g) * 2).half().to(gpu_device),
-             torch.randn(L - 1, hkv, D, generator=g).half().to(gpu_device)) for L in lens]
+    qkv = (torch.randn(B, hq + 2 * hkv, D, generator=g) * 2).to(dtype).to(gpu_device)
+    past = [((torch.randn(L - 1, hkv, D, generator=g) * 2).to(dtype).to(gpu_device),
+             torch.randn(L - 1, hkv, D, generator=g).to(dtype).to(gpu_device)) for L in lens]
     results = []
     for fused in (False, True):
         ctrl = T.make_controller(gpu_device, cap, budget, page_size, batch_size=B, shuffle_seed=3,
-                                 num_heads=hq, num_kv_heads=hkv, scale=scale)
+                                 num_heads=hq, num_kv_heads=hkv, scale=scale, dtype=dtype,
+                                 layout=layout)
         for b, (kk, vv) in enumerate(past):
             if kk.shape[0]:
                 T.fill_sequence(ctrl, kk, vv, seq_idx=b)
@@ -305,7 +310,9 @@ def test_layer_step_equals_append_then_step(gpu_device, lens, hq, hkv, page_size
         for x, y in zip(a, b):
             assert np.array_equal(x.view(np.uint16), y.view(np.uint16))
     assert np.array_equal(np.sort(s0, axis=1), np.sort(s1, axis=1))
-    assert (o0.float() - o1.float()).abs().max().item() <= 1e-3
+    # (bfloat16 outputs are a few units of their last place apart at most: 2^-8 relative)
+    tol = 1e-3 if dtype == torch.float16 else 2e-3 + 2.0 ** -7 * o1.float().abs().max().item()
+    assert (o0.float() - o1.float()).abs().max().item() <= tol
 
 
 @pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 11008), (1008, 520)])
@@ -342,22 +349,28 @@ def test_gemv_add_and_normed_fold_the_residual_and_the_norm(gpu_device, n, k):
 
 
 def test_layer_step_is_refused_where_the_two_launch_step_does_not_apply(gpu_device):
-    """Budgets above 256, bfloat16 and HND pages are served by rope_append_decode + decode_step (or
-    not at all by the decoder operators): the one-call step says so instead of computing something."""
+    """Budgets above 256 are served by rope_append_decode + decode_step: the one-call step says so
+    instead of computing something; and it checks the format of the projection it is given."""
     import adamas_amd.utils as U
     from tests import helpers as T
     cos = torch.ones(1100, 64, device=gpu_device)
     sin = torch.zeros(1100, 64, device=gpu_device)
     qkv = torch.zeros(1, 96, 128, dtype=torch.float16, device=gpu_device)
     kk = torch.zeros(1000, 32, 128, dtype=torch.float16, device=gpu_device)
-    for kwargs, budget in (({}, 512), ({"layout": U.TensorLayout.HND}, 64)):
-        ctrl = T.make_controller(gpu_device, 1100, budget, 16, **kwargs)
-        T.fill_sequence(ctrl, kk, kk)
-        ctrl.prepare_hadamard(1)
-        ctrl.begin_forward(1)
-        assert not U.layer_step_supported(ctrl)
-        with pytest.raises(RuntimeError):
-            U.decode_layer_step(qkv, cos, sin, ctrl, 0)
+    ctrl = T.make_controller(gpu_device, 1100, 512, 16)
+    T.fill_sequence(ctrl, kk, kk)
+    ctrl.prepare_hadamard(1)
+    ctrl.begin_forward(1)
+    assert not U.layer_step_supported(ctrl)
+    with pytest.raises(RuntimeError):
+        U.decode_layer_step(qkv, cos, sin, ctrl, 0)
+    ctrl = T.make_controller(gpu_device, 1100, 64, 16, dtype=torch.bfloat16)
+    T.fill_sequence(ctrl, kk.bfloat16(), kk.bfloat16())
+    ctrl.prepare_hadamard(1)
+    ctrl.begin_forward(1)
+    assert U.layer_step_supported(ctrl)
+    with pytest.raises(RuntimeError):   # a float16 projection for bfloat16 caches
+        U.decode_layer_step(qkv, cos, sin, ctrl, 0)
 
 
 @pytest.mark.parametrize("inter,k", [(11008, 4096), (1002, 264)])
