@@ -8,6 +8,7 @@
 // partial (m, l, o[128]) go to the workspace and the last workgroup to arrive for that head merges
 // them, so there is no second launch.
 #include "attend.h"
+#include "split_merge.h"
 #include "workspace.h"
 
 namespace adamas {
@@ -24,101 +25,13 @@ constexpr uint32_t kDeferredMergeSplits = 24;  // splits from which the partials
 // (measured at 32768 tokens, 32 heads: 16 splits 14.7 us merged inside the launch, 15.8 us with a merge
 // launch; 32 splits 26.6 against 22.5 us)
 
-// Merge of the n_split partial states (m, l, o[128]) of one head, read with agent-scope loads: the
-// values of `kVec` channels starting at channel `ch` for this thread.  kBatch splits are fetched
-// per round (all loads of a round are independent) and folded into a running (M, L, A) with the
-// usual rescaling, so 128 splits cost 128 / kBatch memory round trips instead of 128.
-template <int kVec, int kBatch = 16>
-__device__ __forceinline__ void merge_partials(const float* base, uint32_t n_split, uint32_t ch,
-                                               float& L, float (&A)[kVec]) {
-  float M = kNegBig;
-  L = 0.f;
-#pragma unroll
-  for (int e = 0; e < kVec; ++e) A[e] = 0.f;
-  for (uint32_t s0 = 0; s0 < n_split; s0 += kBatch) {
-    float m[kBatch], l[kBatch], a[kBatch][kVec];
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const uint32_t s2 = min(s0 + u, n_split - 1);  // past the end: a duplicate, weighted zero below
-      const float* p = base + static_cast<size_t>(s2) * kPartialFloats;
-      m[u] = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      l[u] = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-      for (int e = 0; e < kVec; ++e)
-        a[u][e] = __hip_atomic_load(p + 2 + ch + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    float m_new = M;
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) m_new = fmaxf(m_new, s0 + u < n_split ? m[u] : kNegBig);
-    const float keep = exp2_raw(M - m_new);
-    L *= keep;
-#pragma unroll
-    for (int e = 0; e < kVec; ++e) A[e] *= keep;
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const float w = s0 + u < n_split ? exp2_raw(m[u] - m_new) : 0.f;
-      L += l[u] * w;
-#pragma unroll
-      for (int e = 0; e < kVec; ++e) A[e] += a[u][e] * w;
-    }
-    M = m_new;
-  }
-}
-
-// The same for two adjacent channels (ch even) with 64-bit accesses: (m, l) and the channel pair of a
-// partial are each one load, and a thread publishes its pair with one store.
-__device__ __forceinline__ void store_partial_pair(float* p, float a, float b) {
-  const uint64_t v = static_cast<uint64_t>(__float_as_uint(a)) |
-                     (static_cast<uint64_t>(__float_as_uint(b)) << 32);
-  __hip_atomic_store(reinterpret_cast<uint64_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-template <int kBatch>
-__device__ __forceinline__ void merge_partial_pairs(const float* base, uint32_t n_split, uint32_t ch,
-                                                    float& L, float (&A)[2]) {
-  float M = kNegBig;
-  L = 0.f;
-  A[0] = A[1] = 0.f;
-  for (uint32_t s0 = 0; s0 < n_split; s0 += kBatch) {
-    uint64_t ml[kBatch], aa[kBatch];
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const uint32_t s2 = min(s0 + u, n_split - 1);  // past the end: a duplicate, weighted zero below
-      const uint64_t* p =
-          reinterpret_cast<const uint64_t*>(base + static_cast<size_t>(s2) * kPartialFloats);
-      ml[u] = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      aa[u] = __hip_atomic_load(p + 1 + ch / 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    float m_new = M;
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u)
-      m_new = fmaxf(m_new, s0 + u < n_split ? __uint_as_float(static_cast<uint32_t>(ml[u])) : kNegBig);
-    const float keep = exp2_raw(M - m_new);
-    L *= keep;
-    A[0] *= keep;
-    A[1] *= keep;
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const float w = s0 + u < n_split
-                          ? exp2_raw(__uint_as_float(static_cast<uint32_t>(ml[u])) - m_new)
-                          : 0.f;
-      L += __uint_as_float(static_cast<uint32_t>(ml[u] >> 32)) * w;
-      A[0] += __uint_as_float(static_cast<uint32_t>(aa[u])) * w;
-      A[1] += __uint_as_float(static_cast<uint32_t>(aa[u] >> 32)) * w;
-    }
-    M = m_new;
-  }
-}
-
 template <int kGroups>
 struct AttnShared {
   MergeShared<kGroups> merge;
   uint32_t is_last;
 };
 
-// kRowIndex: sel_idx holds K row indices (page * 2 * page_size + slot) instead of token positions;
-// only the row of the current token then goes through the page table.
-template <bool kRowIndex, bool kBf16, bool kHnd, int kThreads = 256>
+template <bool kBf16, bool kHnd, int kThreads = 256>
 __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
     const __half* __restrict__ q, const __half* __restrict__ kv_data,
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
@@ -137,7 +50,7 @@ __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
   const uint32_t bh = b * num_heads + head;
 
   const int32_t seq_len = seq_lens[b];
-  const bool dense = !kRowIndex && sel_idx == nullptr;
+  const bool dense = sel_idx == nullptr;
   const uint32_t n_rows = dense ? static_cast<uint32_t>(seq_len) : n_sel + 1u;
   const int32_t* sel = dense ? nullptr : sel_idx + static_cast<int64_t>(bh) * sel_stride;
   const uint32_t row_begin = split * rows_per_split;
@@ -153,29 +66,14 @@ __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
   kv.seq_len = seq_len;
 
   SoftmaxState st;
-  if (kRowIndex) {
-    int32_t cur_row = -1;  // the current token, last of the list
-    if (seq_len > 0) {
-      const uint32_t p = static_cast<uint32_t>(seq_len - 1);
-      const uint32_t lp = p / page_size;
-      cur_row = static_cast<int32_t>(static_cast<uint32_t>(kv.table[lp]) * kv.row_mult +
-                                     (p - lp * page_size));
-    }
-    attend_rows<kGroups, kTile, true, kBf16, true>(kv, qf, g, row_begin, row_end,
-                                      [&](uint32_t r) __attribute__((always_inline)) -> int32_t {
-                                        return (r < n_sel) ? sel[r] : cur_row;
-                                      },
-                                      st);
-  } else {
-    // (token positions through the page table: branching around unused entries measured faster
-    // here than loading always, 7.9 against 8.0 us at 128 rows)
-    attend_rows<kGroups, kTile, false, kBf16>(kv, qf, g, row_begin, row_end,
-                                [&](uint32_t r) __attribute__((always_inline)) -> int32_t {
-                                  if (dense) return static_cast<int32_t>(r);
-                                  return (r < n_sel) ? sel[r] : seq_len - 1;
-                                },
-                                st);
-  }
+  // (token positions through the page table: branching around unused entries measured faster
+  // here than loading always, 7.9 against 8.0 us at 128 rows)
+  attend_rows<kGroups, kTile, false, kBf16>(kv, qf, g, row_begin, row_end,
+                              [&](uint32_t r) __attribute__((always_inline)) -> int32_t {
+                                if (dense) return static_cast<int32_t>(r);
+                                return (r < n_sel) ? sel[r] : seq_len - 1;
+                              },
+                              st);
 
   float M, L, O;
   merge_groups<kGroups>(st, g, c, tid, sh.merge, M, L, O);
@@ -200,13 +98,7 @@ __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
     }
     return;
   }
-  // ---- several splits: publish the partial, the last arrival merges -----------------------------
-  // The partials cross workgroups inside one launch.  They are written and read with agent-scope
-  // relaxed atomics (write-through stores, cache-bypassing loads) instead of plain accesses fenced
-  // by __threadfence(): an agent-scope fence on this multi-die part writes back and invalidates a
-  // whole L2, once per workgroup.  Every storing wave waits for the acknowledgement of its own
-  // write-through stores (the barrier alone waits for LDS traffic only), then the barrier orders
-  // all of them ahead of the arrival counter that thread 0 bumps.
+  // ---- several splits: publish the partial, the last arrival merges (protocol: split_merge.h) ------
   if (tid < kHeadDim) {
     if (tid == 0) {
       __hip_atomic_store(mine + 0, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -214,14 +106,7 @@ __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
     }
     __hip_atomic_store(mine + 2 + tid, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  wait_own_stores();
-  __syncthreads();
-  if (tid == 0) {
-    const uint32_t prev = atomicAdd(&counters[bh], 1u);
-    sh.is_last = (prev == n_split - 1) ? 1u : 0u;
-  }
-  __syncthreads();
-  if (!sh.is_last) return;
+  if (!split_arrive_is_last(&counters[bh], n_split, sh.is_last, tid)) return;
   if (tid < kHeadDim) {
     float LL, OO[1];
     merge_partials<1>(partial + static_cast<size_t>(bh) * kMaxSplits * kPartialFloats, n_split, tid,
@@ -399,15 +284,8 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_kernel(
   }
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
-  wait_own_stores();
-  __syncthreads();
   uint32_t* counter = counters + static_cast<size_t>(b) * num_heads + hg * kDenseHeads;
-  if (tid == 0) {
-    const uint32_t prev = atomicAdd(counter, 1u);
-    sh.is_last = (prev == n_split - 1) ? 1u : 0u;
-  }
-  __syncthreads();
-  if (!sh.is_last) return;
+  if (!split_arrive_is_last(counter, n_split, sh.is_last, tid)) return;
   {
     float LL, A[2];
     merge_partial_pairs<32>(partial + bh * kMaxSplits * kPartialFloats, n_split, 2 * cp, LL, A);
@@ -579,15 +457,8 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_kernel(
   }
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
-  wait_own_stores();
-  __syncthreads();
   uint32_t* counter = counters + static_cast<size_t>(b) * num_heads + head0;
-  if (tid == 0) {
-    const uint32_t prev = atomicAdd(counter, 1u);
-    sh.is_last = (prev == n_split - 1) ? 1u : 0u;
-  }
-  __syncthreads();
-  if (!sh.is_last) return;
+  if (!split_arrive_is_last(counter, n_split, sh.is_last, tid)) return;
   {
     float LL, A[2];
     merge_partial_pairs<32>(partial + bh * kMaxSplits * kPartialFloats, n_split, 2 * cp, LL, A);
@@ -863,15 +734,8 @@ __global__ __launch_bounds__(kDenseThreads) void dense_decode_gqa_mfma_kernel(
   }
   if (cp == 0) store_partial_pair(mine, M, L);
   store_partial_pair(mine + 2 + 2 * cp, O0, O1);
-  wait_own_stores();
-  __syncthreads();
   uint32_t* counter = counters + static_cast<size_t>(b) * num_heads + head0;
-  if (tid == 0) {
-    const uint32_t prev = atomicAdd(counter, 1u);
-    sh.is_last = (prev == n_split - 1) ? 1u : 0u;
-  }
-  __syncthreads();
-  if (!sh.is_last) return;
+  if (!split_arrive_is_last(counter, n_split, sh.is_last, tid)) return;
   {
     float LL, A[2];
     merge_partial_pairs<32>(partial + bh * kMaxSplits * kPartialFloats, n_split, 2 * cp, LL, A);
@@ -890,18 +754,16 @@ extern "C" size_t adamas_workspace_bytes(uint32_t batch, uint32_t num_heads, uin
   return workspace_layout(batch, num_heads, max_seq_len, budget).total;
 }
 
-// sel_is_rows: sel_idx holds K row indices instead of token positions (never null then)
 static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t* page_indices,
                               const int32_t* page_indptr, const int32_t* seq_lens,
                               const int32_t* sel_idx, int64_t sel_stride, uint32_t n_sel, void* out,
                               void* workspace, size_t workspace_bytes, uint32_t batch,
                               uint32_t num_heads, uint32_t num_kv_heads, uint32_t head_dim,
                               uint32_t page_size, float sm_scale, uint32_t max_seq_len,
-                              adamas_stream_t stream, bool sel_is_rows, uint32_t flags) {
+                              adamas_stream_t stream, uint32_t flags) {
   if (flags & ~(ADAMAS_F_BF16 | ADAMAS_F_HND | ADAMAS_F_NO_MFMA)) return ADAMAS_E_BADARG;
   const bool bf16 = (flags & ADAMAS_F_BF16) != 0;
   const KvLayout lay = make_kv_layout((flags & ADAMAS_F_HND) != 0, page_size, num_kv_heads);
-  if (sel_is_rows && !sel_idx) return ADAMAS_E_BADARG;
   if (!q || !kv_data || !page_indices || !page_indptr || !seq_lens || !out || batch == 0 ||
       num_heads == 0 || page_size == 0 || max_seq_len == 0)
     return ADAMAS_E_BADARG;
@@ -1038,37 +900,29 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
   }
   // from kDeferredMergeSplits splits on, the merge is a second short launch
   const uint32_t deferred = n_split >= kDeferredMergeSplits ? 1u : 0u;
-#define ADAMAS_LAUNCH_SPARSE_T(ROWS, BF, HND, T)                                                 \
-  hipLaunchKernelGGL((sparse_decode_kernel<ROWS, BF, HND, T>), dim3(n_split, num_heads, batch),  \
+#define ADAMAS_LAUNCH_SPARSE_T(BF, HND, T)                                                       \
+  hipLaunchKernelGGL((sparse_decode_kernel<BF, HND, T>), dim3(n_split, num_heads, batch),        \
                      dim3(T), 0, static_cast<hipStream_t>(stream),                               \
                      static_cast<const __half*>(q), static_cast<const __half*>(kv_data),         \
                      page_indices, page_indptr, seq_lens, sel_idx, sel_stride, n_sel,            \
                      static_cast<__half*>(out), partial, counters, num_heads, num_kv_heads,      \
                      page_size, scale_log2, rows_per_split, deferred)
-#define ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, HND)       \
-  if (wide) {                                       \
-    ADAMAS_LAUNCH_SPARSE_T(ROWS, BF, HND, 512);     \
-  } else {                                          \
-    ADAMAS_LAUNCH_SPARSE_T(ROWS, BF, HND, 256);     \
-  }
-#define ADAMAS_LAUNCH_SPARSE(ROWS, BF)        \
-  if (flags & ADAMAS_F_HND) {                 \
-    ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, true)    \
+#define ADAMAS_LAUNCH_SPARSE_L(BF, HND)       \
+  if (wide) {                                 \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512);     \
   } else {                                    \
-    ADAMAS_LAUNCH_SPARSE_L(ROWS, BF, false)   \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 256);     \
   }
-  if (sel_is_rows) {
-    if (bf16) {
-      ADAMAS_LAUNCH_SPARSE(true, true)
-    } else {
-      ADAMAS_LAUNCH_SPARSE(true, false)
-    }
+#define ADAMAS_LAUNCH_SPARSE(BF)        \
+  if (flags & ADAMAS_F_HND) {           \
+    ADAMAS_LAUNCH_SPARSE_L(BF, true)    \
+  } else {                              \
+    ADAMAS_LAUNCH_SPARSE_L(BF, false)   \
+  }
+  if (bf16) {
+    ADAMAS_LAUNCH_SPARSE(true)
   } else {
-    if (bf16) {
-      ADAMAS_LAUNCH_SPARSE(false, true)
-    } else {
-      ADAMAS_LAUNCH_SPARSE(false, false)
-    }
+    ADAMAS_LAUNCH_SPARSE(false)
   }
 #undef ADAMAS_LAUNCH_SPARSE
 #undef ADAMAS_LAUNCH_SPARSE_L
@@ -1098,7 +952,7 @@ extern "C" int adamas_sparse_decode_f(const void* q, const void* kv_data,
                                       uint32_t flags, adamas_stream_t stream) {
   return sparse_decode_impl(q, kv_data, page_indices, page_indptr, seq_lens, sel_idx, sel_stride,
                             n_sel, out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
-                            head_dim, page_size, sm_scale, max_seq_len, stream, false, flags);
+                            head_dim, page_size, sm_scale, max_seq_len, stream, flags);
 }
 
 extern "C" int adamas_sparse_decode(const void* q, const void* kv_data,
@@ -1110,20 +964,7 @@ extern "C" int adamas_sparse_decode(const void* q, const void* kv_data,
                                     float sm_scale, uint32_t max_seq_len, adamas_stream_t stream) {
   return sparse_decode_impl(q, kv_data, page_indices, page_indptr, seq_lens, sel_idx, sel_stride,
                             n_sel, out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
-                            head_dim, page_size, sm_scale, max_seq_len, stream, false, 0u);
-}
-
-int adamas::launch_sparse_decode_rows(const void* q, const void* kv_data,
-                                      const int32_t* page_indices, const int32_t* page_indptr,
-                                      const int32_t* seq_lens, const int32_t* sel_rows,
-                                      int64_t sel_stride, uint32_t n_sel, void* out,
-                                      void* workspace, size_t workspace_bytes, uint32_t batch,
-                                      uint32_t num_heads, uint32_t num_kv_heads, uint32_t head_dim,
-                                      uint32_t page_size, float sm_scale, uint32_t max_seq_len,
-                                      uint32_t flags, hipStream_t stream) {
-  return sparse_decode_impl(q, kv_data, page_indices, page_indptr, seq_lens, sel_rows, sel_stride,
-                            n_sel, out, workspace, workspace_bytes, batch, num_heads, num_kv_heads,
-                            head_dim, page_size, sm_scale, max_seq_len, stream, true, flags);
+                            head_dim, page_size, sm_scale, max_seq_len, stream, 0u);
 }
 
 extern "C" int adamas_version(void) { return 100; }

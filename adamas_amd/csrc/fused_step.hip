@@ -31,6 +31,7 @@
 #include <atomic>
 
 #include "chunk_select.h"
+#include "split_merge.h"
 #include "workspace.h"
 
 namespace adamas {
@@ -137,9 +138,9 @@ __device__ __forceinline__ uint32_t wave_query_code(const WaveRopeLoads& r, int 
 // kHist (budgets beyond the candidate lists, chunks of 512 tokens): instead of selecting, every wave
 // writes the distances of its head (dist_out [sequence*heads][dist_stride] u16) and a 512-bin
 // histogram of them (16-bit counts, hist_out [sequence*heads][chunks][512]); threshold and positions
-// are then read off the histograms by the integer top-k (topk.hip).  The first head group also
-// writes the K row index of every token (rowmap_out [sequence][dist_stride]), so that the selection
-// can hand row indices to the attention, which then reads no page table.
+// are then read off the histograms by hist_select_attend_kernel below.  The first head group also
+// writes the K row index of every token (rowmap_out [sequence][dist_stride]), so that the attention
+// of that kernel reads no page table.
 // kFromQkv: q_code is not read; wave w makes the code of query head w of the group from the fused
 // projection (rotary embedding, Hadamard transform, buckets) while the code loads are in flight.
 // qcode_out (selection mode) [sequence*heads][16]: the query codes this launch worked with, written by
@@ -781,6 +782,271 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   if (tid < kHeadDim) store_elem<kBf16>(out + static_cast<size_t>(bh) * kHeadDim + tid, O / L);
 }
 
+// ---- budgets beyond the candidate lists: selection from the histograms and attention in one launch --
+// The estimator in histogram mode leaves, per head, the distances of all tokens, a 512-bin histogram
+// per chunk of 512 tokens and, per sequence, the K row index of every token.  grid (sequence*heads,
+// slabs of 4096 tokens), 256 threads.  Every workgroup works the threshold out for itself from the
+// chunk rows (they are small and sit in L2; rows of one head are the fast grid dimension so that its
+// slabs share a die), adding up on the side the rows of the chunks BEFORE its slab: those give the
+// number of selected tokens that precede the slab, i.e. the tie quota left for it and where its
+// positions go.  Then it selects among its own 4096 distances (class masks and DPP prefix scans),
+// keeps the K rows of the selected tokens in LDS and attends them: 16 groups of 16 lanes, tiles of
+// 8 rows.  The slabs of a head are merged inside the launch (split_merge.h).  Against a launch that
+// writes the selection followed by the attention operator, this saves a launch, the list's trip
+// through memory and the wait for it.
+constexpr int kHsaThreads = 256;
+constexpr int kHsaWaves = kHsaThreads / kWave;
+constexpr int kHsaItems = 16;                                    // distances per thread
+constexpr uint32_t kHsaSlab = kHsaThreads * kHsaItems;           // 4096 tokens per workgroup
+constexpr uint32_t kHsaSlabChunks = kHsaSlab / kFusedBlock;      // 8 histogram rows per slab
+constexpr int kHsaGroups = kHsaThreads / 16;
+constexpr uint32_t kHsaMaxTokens = kHsaSlab * 32;                // 32 slabs per head at most
+
+struct HistSelectAttendShared {
+  alignas(16) uint32_t all[kHsaWaves][kHistBins];  // partial sums over all chunk rows
+  alignas(16) uint32_t pre[kHsaWaves][kHistBins];  // partial sums over the chunk rows before the slab
+  uint32_t wtot[kHsaWaves], wpre[kHsaWaves], wclass[kHsaWaves];
+  uint32_t pre_tied;   // tokens at the threshold distance in the chunks before the slab
+  SelectPlan plan;
+  int32_t rows[kHsaSlab + 1];  // K rows of the slab's selected tokens (slab 0: then the current token)
+  MergeShared<kHsaGroups> merge;
+  uint32_t is_last;
+};
+
+template <bool kBf16, bool kHnd>
+__global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
+    const __half* __restrict__ q, const __half* __restrict__ kv_data,
+    const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
+    const int32_t* __restrict__ seq_lens, const uint16_t* __restrict__ dist, int64_t dist_stride,
+    const uint16_t* __restrict__ hist, uint32_t n_chunks, const uint32_t* __restrict__ rowmap,
+    uint32_t k, __half* __restrict__ out, int32_t* __restrict__ sel_out, float* partial,
+    uint32_t* __restrict__ counters, uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_inv16,
+    uint32_t page_size, float scale_log2) {
+  static_assert(kHsaThreads * 2 == kHistBins, "two bins per thread in the prefix sum");
+  __shared__ HistSelectAttendShared sh;
+  const uint32_t bh = blockIdx.x, slab = blockIdx.y;
+  const uint32_t b = bh / num_heads, head = bh - b * num_heads;
+  const uint32_t tid = threadIdx.x;
+  const int lane = lane_id();
+  const int wave = wave_id_uniform();
+  const uint32_t g = tid >> 4, c16 = tid & 15;
+  int32_t* sdst = sel_out ? sel_out + static_cast<size_t>(bh) * k : nullptr;
+  const int32_t seq_len = seq_lens[b];
+  if (seq_len <= 0) {  // a sequence without tokens: zeros and an empty selection
+    if (slab == 0) {
+      if (tid < kHeadDim) store_elem<kBf16>(out + static_cast<size_t>(bh) * kHeadDim + tid, 0.f);
+      if (sdst)
+        for (uint32_t i = tid; i < k; i += kHsaThreads) sdst[i] = -1;
+    }
+    return;
+  }
+  const uint32_t n = static_cast<uint32_t>(seq_len) - 1u;                 // past tokens
+  const uint32_t n_split = n ? (n + kHsaSlab - 1) / kHsaSlab : 1u;        // slabs that hold tokens
+  if (slab >= n_split) return;
+  const uint32_t slab_base = slab * kHsaSlab;
+  // thread t holds the 16 consecutive tokens t*16 .. t*16+15 of the slab: distances and K rows,
+  // asked for first
+  const uint32_t e0 = slab_base + tid * kHsaItems;
+  uint32_t keys[kHsaItems], trow[kHsaItems];
+  {
+    const uint16_t* vrow = dist + static_cast<int64_t>(bh) * dist_stride + e0;  // 16-byte aligned
+    const uint32_t* rm = rowmap + static_cast<int64_t>(b) * dist_stride + e0;
+    uint4 kraw[2], rraw[4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      kraw[j] = e0 + 8 * j < n ? *reinterpret_cast<const uint4*>(vrow + 8 * j)
+                               : make_uint4(~0u, ~0u, ~0u, ~0u);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      rraw[j] = e0 + 4 * j < n ? *reinterpret_cast<const uint4*>(rm + 4 * j)
+                               : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t w[4] = {kraw[j].x, kraw[j].y, kraw[j].z, kraw[j].w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t v = (w[i >> 1] >> (16 * (i & 1))) & 0xffffu;
+        keys[8 * j + i] = e0 + 8 * j + i < n ? v : 0xffffu;  // past the end: above every threshold
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      trow[4 * j] = rraw[j].x;
+      trow[4 * j + 1] = rraw[j].y;
+      trow[4 * j + 2] = rraw[j].z;
+      trow[4 * j + 3] = rraw[j].w;
+    }
+  }
+  float qf[8];
+  load_query<kBf16>(q + static_cast<size_t>(bh) * kHeadDim, c16, scale_log2, qf);
+  const int32_t* table = page_indices + page_indptr[b];
+  const uint32_t rows_per_page = kHnd ? 2u * page_size * num_kv_heads : 2u * page_size;
+  int32_t cur_row = 0;
+  if (slab == 0) {  // the current token is attended with the first slab
+    const uint32_t lp = n / page_size;
+    cur_row = static_cast<int32_t>(static_cast<uint32_t>(table[lp]) * rows_per_page + (n - lp * page_size));
+  }
+
+  // ---- chunk rows (16-bit counts): thread (part, seg) adds bins 8*seg .. 8*seg+7 of rows part, part+4, ...
+  {
+    const uint32_t part = tid >> 6, seg = tid & 63u;
+    const uint32_t c_first = slab * kHsaSlabChunks;  // chunks below it precede the slab
+    const unsigned char* hb = reinterpret_cast<const unsigned char*>(hist) +
+                              static_cast<size_t>(bh) * n_chunks * (2 * kHistBins) + seg * 16u;
+    const uint32_t rows_used = min(n_chunks, (n + kFusedBlock - 1) / kFusedBlock);  // rows of this sequence
+    uint32_t acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, pre[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (uint32_t c0 = part; c0 < rows_used; c0 += 16) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t c = c0 + 4u * u;
+        v[u] = c < rows_used
+                   ? *reinterpret_cast<const uint4*>(hb + static_cast<size_t>(c) * (2 * kHistBins))
+                   : make_uint4(0u, 0u, 0u, 0u);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+        const uint32_t m = (c0 + 4u * u < c_first) ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[2 * j] += w[j] & 0xffffu;
+          acc[2 * j + 1] += w[j] >> 16;
+          pre[2 * j] += w[j] & 0xffffu & m;
+          pre[2 * j + 1] += (w[j] >> 16) & m;
+        }
+      }
+    }
+    uint4* da = reinterpret_cast<uint4*>(&sh.all[part][seg * 8u]);
+    da[0] = make_uint4(acc[0], acc[1], acc[2], acc[3]);
+    da[1] = make_uint4(acc[4], acc[5], acc[6], acc[7]);
+    uint4* dp = reinterpret_cast<uint4*>(&sh.pre[part][seg * 8u]);
+    dp[0] = make_uint4(pre[0], pre[1], pre[2], pre[3]);
+    dp[1] = make_uint4(pre[4], pre[5], pre[6], pre[7]);
+  }
+  __syncthreads();
+  // ---- thread t owns bins 2t and 2t+1: prefix sum -> the plan
+  uint32_t ca0 = 0, ca1 = 0, cp0 = 0, cp1 = 0;
+#pragma unroll
+  for (int p = 0; p < kHsaWaves; ++p) {
+    const uint2 x = *reinterpret_cast<const uint2*>(&sh.all[p][2 * tid]);
+    const uint2 y = *reinterpret_cast<const uint2*>(&sh.pre[p][2 * tid]);
+    ca0 += x.x;
+    ca1 += x.y;
+    cp0 += y.x;
+    cp1 += y.y;
+  }
+  const uint32_t incl = wave_inclusive_scan_dpp(ca0 + ca1);
+  if (lane == kWave - 1) sh.wtot[wave] = incl;
+  __syncthreads();
+  uint32_t cum1 = incl;  // tokens with a distance <= bin 2t+1
+  for (int w = 0; w < wave; ++w) cum1 += sh.wtot[w];
+  const uint32_t cum0 = cum1 - ca1;  // <= bin 2t
+  if (cum0 >= k && cum0 - ca0 < k) {  // exactly one bin holds the k-th smallest distance
+    sh.plan.thr = 2 * tid;
+    sh.plan.n_below = cum0 - ca0;
+    sh.plan.quota = k - (cum0 - ca0);
+    sh.plan.n_take = k;
+    sh.pre_tied = cp0;
+  }
+  if (cum1 >= k && cum0 < k) {
+    sh.plan.thr = 2 * tid + 1;
+    sh.plan.n_below = cum0;
+    sh.plan.quota = k - cum0;
+    sh.plan.n_take = k;
+    sh.pre_tied = cp1;
+  }
+  if (tid == kHsaThreads - 1 && cum1 < k) {  // fewer tokens than k: all of them are taken
+    sh.plan.thr = kHistBins;
+    sh.plan.n_below = cum1;
+    sh.plan.quota = 0;
+    sh.plan.n_take = cum1;
+    sh.pre_tied = 0;
+  }
+  __syncthreads();
+  const SelectPlan plan = sh.plan;
+  const uint32_t pre_tied = sh.pre_tied;
+
+  // ---- selected tokens before the slab, class masks and ranks inside it
+  const uint32_t mine_pre = (2 * tid < plan.thr ? cp0 : 0u) + (2 * tid + 1 < plan.thr ? cp1 : 0u);
+  const uint32_t wave_pre = wave_sum(mine_pre);
+  uint32_t below[kHsaItems / 4], equal[kHsaItems / 4];
+  raw_class_masks<kHsaItems>(keys, plan.thr, below, equal);
+  uint32_t total;
+  const uint32_t excl = lane_scan<kHsaItems / 4>(below, equal, total);  // below | tied << 16
+  if (lane == 0) {
+    sh.wpre[wave] = wave_pre;
+    sh.wclass[wave] = total;
+  }
+  __syncthreads();
+  uint32_t base_b = 0, before = 0, slab_all = 0;
+#pragma unroll
+  for (int w = 0; w < kHsaWaves; ++w) {
+    base_b += sh.wpre[w];
+    before += w < wave ? sh.wclass[w] : 0u;
+    slab_all += sh.wclass[w];
+  }
+  const uint32_t slab_below = slab_all & 0xffffu, slab_tied = slab_all >> 16;
+  // tied tokens of this slab that are inside the quota (ties go to the lowest index: the chunks
+  // before the slab come first)
+  const uint32_t tied_left = plan.quota > pre_tied ? plan.quota - pre_tied : 0u;
+  const uint32_t slab_tied_taken = min(slab_tied, tied_left);
+  // positions in the whole selection: the tokens below the threshold in index order, then the ties
+  lane_emit<kHsaItems / 4>(below, equal, plan.n_below, plan.quota,
+                           base_b + (before & 0xffffu) + (excl & 0xffffu),
+                           pre_tied + (before >> 16) + (excl >> 16),
+                           [&](uint32_t pos, int i) __attribute__((always_inline)) {
+                             const bool is_b = keys[i] < plan.thr;
+                             const uint32_t local = is_b ? pos - base_b
+                                                         : slab_below + (pos - plan.n_below - pre_tied);
+                             sh.rows[local] = static_cast<int32_t>(trow[i]);
+                             if (sdst) sdst[pos] = static_cast<int32_t>(e0 + i);
+                           });
+  uint32_t n_rows = slab_below + slab_tied_taken;
+  if (slab == 0) {
+    if (tid == 0) sh.rows[n_rows] = cur_row;
+    ++n_rows;
+    if (sdst)
+      for (uint32_t i = plan.n_take + tid; i < k; i += kHsaThreads) sdst[i] = -1;
+  }
+  __syncthreads();
+
+  // ---- attention over the rows of the slab -------------------------------------------------------------
+  HeadKV kv;
+  kv.kv_data = kv_data;
+  kv.table = nullptr;  // rows are K row indices already
+  set_kv_layout_static<kHnd>(kv, kv_head_of(head, kv_inv16), c16, num_kv_heads, page_size);
+  kv.seq_len = seq_len;
+  SoftmaxState st;
+  attend_rows<kHsaGroups, 8, true, kBf16, true>(
+      kv, qf, g, 0u, n_rows,
+      [&](uint32_t r) __attribute__((always_inline)) -> int32_t { return sh.rows[r]; }, st);
+  float M, L, O;
+  merge_groups<kHsaGroups>(st, g, c16, tid, sh.merge, M, L, O);
+  if (n_split == 1) {
+    if (tid < kHeadDim)
+      store_elem<kBf16>(out + static_cast<size_t>(bh) * kHeadDim + tid, L > 0.f ? O / L : 0.f);
+    return;
+  }
+  // several slabs: publish the partial, the last arrival merges (protocol: split_merge.h)
+  float* mine = partial + (static_cast<size_t>(bh) * kMaxSplits + slab) * kPartialFloats;
+  if (tid < kHeadDim) {
+    if (tid == 0) {
+      __hip_atomic_store(mine + 0, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(mine + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __hip_atomic_store(mine + 2 + tid, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (!split_arrive_is_last(&counters[bh], n_split, sh.is_last, tid)) return;
+  if (tid < kHeadDim) {
+    float LL, OO[1];
+    merge_partials<1>(partial + static_cast<size_t>(bh) * kMaxSplits * kPartialFloats, n_split, tid,
+                      LL, OO);
+    store_elem<kBf16>(out + static_cast<size_t>(bh) * kHeadDim + tid, LL > 0.f ? OO[0] / LL : 0.f);
+  }
+  if (tid == 0) counters[bh] = 0;  // ready for the next launch on this stream
+}
+
 }  // namespace adamas
 
 using namespace adamas;
@@ -1067,8 +1333,8 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
   uint16_t* dist = reinterpret_cast<uint16_t*>(ws + w.dist_off);
   int32_t* sel = sel_out ? sel_out : reinterpret_cast<int32_t*>(ws + w.sel_off);
   // budgets beyond the candidate lists, rows of moderate length: the estimator writes the distances
-  // and a histogram per 512-token chunk, the selection reads threshold and positions off the
-  // histograms, then the attention over the selected tokens (three launches)
+  // and a histogram per 512-token chunk; the second launch reads threshold and positions off the
+  // histograms and attends the selected tokens (also two launches)
   if (n_sel > 0 && max_seq_len > 1 && max_seq_len - 1 <= 131072 && w.hist_stride > 0 &&
       batch <= 65535) {
     // workgroups of 4 heads wherever the 8-head ones would leave CUs idle or unevenly loaded
@@ -1087,7 +1353,6 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
     unsigned char* hist = reinterpret_cast<unsigned char*>(ws + w.hist_off);
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint32_t* rowmap = reinterpret_cast<uint32_t*>(ws + w.rowmap_off);
-    int32_t* sel_rows = reinterpret_cast<int32_t*>(ws + w.rows_off);
 #define ADAMAS_LAUNCH_ESTHIST_H(PG, HEADS)                                                       \
   hipLaunchKernelGGL((estimate_select_kernel<PG, 1, false, true, HEADS>), grid,                  \
                      dim3(HEADS * kWave), 0, s,                                                  \
@@ -1113,15 +1378,31 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
 #undef ADAMAS_LAUNCH_ESTHIST
 #undef ADAMAS_LAUNCH_ESTHIST_H
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
-    const int rc = launch_hist_select(dist, w.dist_stride, max_seq_len - 1, seq_lens, num_heads,
-                                      batch * num_heads, n_sel, sel, static_cast<int64_t>(n_sel),
-                                      reinterpret_cast<const uint16_t*>(hist), w.hist_stride,
-                                      kFusedBlock, rowmap, w.dist_stride, sel_rows, s);
-    if (rc != 0) return rc;
-    return launch_sparse_decode_rows(q, kv_data, page_indices, page_indptr, seq_lens, sel_rows,
-                                     static_cast<int64_t>(n_sel), n_sel, out, workspace,
-                                     workspace_bytes, batch, num_heads, num_kv_heads, head_dim,
-                                     page_size, sm_scale, max_seq_len, flags, s);
+    // selection from the histograms and attention over the selected rows, one launch
+    const bool bf16 = (flags & ADAMAS_F_BF16) != 0, hnd = (flags & ADAMAS_F_HND) != 0;
+    const dim3 hgrid(batch * num_heads, (max_seq_len - 1 + kHsaSlab - 1) / kHsaSlab);
+#define ADAMAS_LAUNCH_HSA(BF, HND)                                                                 \
+  hipLaunchKernelGGL((hist_select_attend_kernel<BF, HND>), hgrid, dim3(kHsaThreads), 0, s,         \
+                     static_cast<const __half*>(q), static_cast<const __half*>(kv_data),           \
+                     page_indices, page_indptr, seq_lens, dist, w.dist_stride,                     \
+                     reinterpret_cast<const uint16_t*>(hist), w.hist_stride, rowmap, n_sel,        \
+                     static_cast<__half*>(out), sel_out,                                           \
+                     reinterpret_cast<float*>(ws + w.partial_off),                                 \
+                     reinterpret_cast<uint32_t*>(ws + w.counters_off), num_heads, num_kv_heads,    \
+                     group_inv16(num_heads / num_kv_heads), page_size,                             \
+                     sm_scale * 1.4426950408889634f)
+    if (bf16 && hnd) {
+      ADAMAS_LAUNCH_HSA(true, true);
+    } else if (bf16) {
+      ADAMAS_LAUNCH_HSA(true, false);
+    } else if (hnd) {
+      ADAMAS_LAUNCH_HSA(false, true);
+    } else {
+      ADAMAS_LAUNCH_HSA(false, false);
+    }
+#undef ADAMAS_LAUNCH_HSA
+    ADAMAS_RETURN_IF_LAUNCH_FAILED();
+    return 0;
   }
   // general path: the stand-alone entry points one after the other
   if (n_sel > 0 && max_seq_len > 1) {

@@ -54,11 +54,6 @@ struct SelectArgs {
   int32_t* out_idx;
   uint16_t* out_vals;
   int64_t out_stride;
-  // optional (histogram emission): K row index of every token of a sequence, and where the row
-  // indices of the selected tokens go (laid out like out_idx)
-  const uint32_t* rowmap;
-  int64_t rowmap_stride;
-  int32_t* out_rows;
 };
 
 __device__ __forceinline__ uint32_t row_length(const SelectArgs& a, uint32_t row) {
@@ -621,22 +616,6 @@ __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
   for (int j = 0; j < kEmitItems / 8; ++j)
     load_value_keys<kPadded>(vrow, e0 + j * 8, n, vec_ok, key_mode, &keys[j * 8]);
 
-  // the K row indices of the same 16 tokens, when asked for (16-byte aligned: rows of the map are)
-  int32_t* rdst = a.out_rows ? a.out_rows + static_cast<int64_t>(row) * a.out_stride : nullptr;
-  uint32_t trow[kEmitItems];
-  if (rdst) {
-    const uint32_t* rm = a.rowmap + static_cast<int64_t>(row / a.rows_per_seq) * a.rowmap_stride + e0;
-#pragma unroll
-    for (int j = 0; j < kEmitItems / 4; ++j) {
-      const uint4 t = (e0 + 4 * j < n) ? *reinterpret_cast<const uint4*>(rm + 4 * j)
-                                       : make_uint4(0u, 0u, 0u, 0u);
-      trow[4 * j] = t.x;
-      trow[4 * j + 1] = t.y;
-      trow[4 * j + 2] = t.z;
-      trow[4 * j + 3] = t.w;
-    }
-  }
-
   // ---- chunk rows: thread (part, seg) adds bins 8*seg .. 8*seg+7 of rows part, part + 4, ...
   {
     const uint32_t part = tid >> 6, seg = tid & 63u;
@@ -739,7 +718,6 @@ __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
                             [&](uint32_t pos, int i) __attribute__((always_inline)) {
                               const uint32_t e = e0 + i;
                               idst[pos] = grow ? grow[e] : static_cast<int32_t>(e);
-                              if (rdst) rdst[pos] = static_cast<int32_t>(trow[i]);
                               if (vdst)
                                 vdst[pos] =
                                     static_cast<uint16_t>(raw_of_key(keys[i], key_mode));
@@ -747,49 +725,9 @@ __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
   if (slab == 0) {
     for (uint32_t i = plan.n_take + tid; i < k; i += kEmitThreads) {
       idst[i] = -1;
-      if (rdst) rdst[i] = -1;
       if (vdst) vdst[i] = 0;
     }
   }
-}
-
-// Selection from histograms that another kernel has written (the estimator of the decode step for
-// large budgets: chunks of `chunk_keys` = 512 keys): positions of the k smallest u16 distances of
-// every row into out_idx.  Rows are [sequence][head] with lengths seq_lens[row / rows_per_seq] - 1.
-int launch_hist_select(const uint16_t* dist, int64_t row_stride, uint32_t n_max,
-                       const int32_t* seq_lens, uint32_t rows_per_seq, uint32_t num_rows,
-                       uint32_t k, int32_t* out_idx, int64_t out_stride, const uint16_t* hist,
-                       uint32_t n_chunks, uint32_t chunk_keys, const uint32_t* rowmap,
-                       int64_t rowmap_stride, int32_t* out_rows, hipStream_t stream) {
-  if (n_max > kEmitMaxRowLen || kEmitSlab % chunk_keys != 0) return ADAMAS_E_UNSUPPORTED;
-  if (out_rows && (!rowmap || rowmap_stride % 4 != 0 ||
-                   (reinterpret_cast<uintptr_t>(rowmap) & 15) != 0))
-    return ADAMAS_E_ALIGN;
-  SelectArgs a{};
-  a.values = dist;
-  a.row_stride = row_stride;
-  a.n_max = n_max;
-  a.seq_lens = seq_lens;
-  a.rows_per_seq = rows_per_seq;
-  a.len_delta = -1;
-  a.vec_ok = ((reinterpret_cast<uintptr_t>(dist) & 15) == 0 && row_stride % 8 == 0) ? 1u : 0u;
-  a.k = k;
-  a.key_mode = ADAMAS_KEY_U16_INT;
-  a.out_idx = out_idx;
-  a.out_stride = out_stride;
-  a.rowmap = rowmap;
-  a.rowmap_stride = rowmap_stride;
-  a.out_rows = out_rows;
-  // the distance rows of the step's workspace are aligned and padded to a multiple of 8 elements
-  if (a.vec_ok && row_stride >= static_cast<int64_t>((n_max + 7) / 8 * 8))
-    hipLaunchKernelGGL((select_hist_emit_kernel<ADAMAS_KEY_U16_INT, true>),
-                       dim3(num_rows, ceil_div(n_max, kEmitSlab)), dim3(kEmitThreads), 0, stream, a,
-                       hist, n_chunks, kEmitSlab / chunk_keys);
-  else
-    hipLaunchKernelGGL(select_hist_emit_kernel<-1>, dim3(num_rows, ceil_div(n_max, kEmitSlab)),
-                       dim3(kEmitThreads), 0, stream, a, hist, n_chunks, kEmitSlab / chunk_keys);
-  ADAMAS_RETURN_IF_LAUNCH_FAILED();
-  return 0;
 }
 
 static size_t hist_path_bytes(uint32_t num_rows, uint32_t n_max) {

@@ -122,8 +122,6 @@ struct WorkspaceLayout {
   size_t dist_off;      // uint16 [batch*heads][dist_stride]: distances of the step for large budgets;
                         // in the two-launch step, the re-scored distances of truncated chunks
   size_t sel_off;       // int32  [batch*heads][budget], selection of the fused step
-  size_t rows_off;      // int32  [batch*heads][budget], K row index of every selected token (the step
-                        // for large budgets: the attention then needs no page-table access)
   size_t rowmap_off;    // uint32 [batch][dist_stride], K row index of every past token (same step)
   size_t topk_off;      // workspace of adamas_topk inside the fused step
   size_t topk_bytes;
@@ -153,8 +151,6 @@ inline WorkspaceLayout workspace_layout(uint32_t batch, uint32_t num_heads, uint
   off = align_up(off + rows * static_cast<size_t>(w.dist_stride) * sizeof(uint16_t), 256);
   w.sel_off = off;
   off = align_up(off + rows * static_cast<size_t>(budget ? budget : 1) * sizeof(int32_t), 256);
-  w.rows_off = off;
-  off = align_up(off + rows * static_cast<size_t>(budget ? budget : 1) * sizeof(int32_t), 256);
   w.rowmap_off = off;
   off = align_up(off + static_cast<size_t>(batch) * static_cast<size_t>(w.dist_stride) * sizeof(uint32_t), 256);
   w.topk_off = off;
@@ -180,24 +176,5 @@ inline WorkspaceLayout workspace_layout(uint32_t batch, uint32_t num_heads, uint
   w.total = off;
   return w;
 }
-
-// topk.hip: selection from chunk histograms written by the estimator (see there)
-// rowmap (optional) [sequence][rowmap_stride]: K row index of every token; out_rows then receives the
-// K row index of every selected token, laid out like out_idx.
-int launch_hist_select(const uint16_t* dist, int64_t row_stride, uint32_t n_max,
-                       const int32_t* seq_lens, uint32_t rows_per_seq, uint32_t num_rows,
-                       uint32_t k, int32_t* out_idx, int64_t out_stride, const uint16_t* hist,
-                       uint32_t n_chunks, uint32_t chunk_keys, const uint32_t* rowmap,
-                       int64_t rowmap_stride, int32_t* out_rows, hipStream_t stream);
-
-// attention.hip: adamas_sparse_decode_f over a list of K row indices (page * rows per page + slot,
-// negative = skip) instead of token positions: no page-table access per row
-int launch_sparse_decode_rows(const void* q, const void* kv_data, const int32_t* page_indices,
-                              const int32_t* page_indptr, const int32_t* seq_lens,
-                              const int32_t* sel_rows, int64_t sel_stride, uint32_t n_sel,
-                              void* out, void* workspace, size_t workspace_bytes, uint32_t batch,
-                              uint32_t num_heads, uint32_t num_kv_heads, uint32_t head_dim,
-                              uint32_t page_size, float sm_scale, uint32_t max_seq_len,
-                              uint32_t flags, hipStream_t stream);
 
 }  // namespace adamas

@@ -250,7 +250,7 @@ int adamas_sparse_decode_f(const void* q, const void* kv_data, const int32_t* pa
  * starts at page_indices[b * page_table_stride] (fixed-stride tables), every entry of a row must be
  * a valid page id, and the kernels fetch page ids and sequence length side by side instead of one
  * after the other (one memory round trip less per launch).  page_indptr is still required here
- * (the three-launch path uses it); the two functions below accept NULL with a non-zero stride.
+ * (the paths for larger budgets use it); the two functions below accept NULL with a non-zero stride.
  * Replaces the call sequence decode_estimate / decode_topk / decode_sparse_attn of
  * adamas/models/Adamas.py:176-201 (adamas/utils/__init__.py:203-308).
  */
@@ -295,8 +295,11 @@ int adamas_decode_step_noalloc(const void* q, const void* q_code, const void* kv
  * The two halves of adamas_decode_step, for callers that want to time or schedule them separately.
  * adamas_step_fused_supported returns 1 when these sizes are served by the two-launch path (budget
  * <= 256; one sequence of up to 131072 tokens, or several whose chunk lists fit: at most 64 chunks of
- * 512, 1024 or 2048 tokens each); otherwise adamas_decode_step runs estimate, top-k and attention as
- * three launches and the two functions below return ADAMAS_E_UNSUPPORTED.
+ * 512, 1024 or 2048 tokens each); otherwise adamas_decode_step takes another route (budgets above
+ * 256 on rows of up to 131072 tokens: an estimator launch that leaves distances and per-chunk
+ * histograms, and a launch that selects from the histograms and attends; anything else: the three
+ * stand-alone operators one after the other) and the two functions below return
+ * ADAMAS_E_UNSUPPORTED.
  *   adamas_step_candidates : distance estimate over the code cache fused with the selection of the
  *                            nearest tokens of every chunk (chunks of a single sequence are balanced:
  *                            their lengths differ by at most 16 tokens and their number does not
