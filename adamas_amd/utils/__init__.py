@@ -356,6 +356,15 @@ class BatchDecodeWithPagedKVCacheWrapper:
             # (decode_handler.cuh:226-231)
             raise RuntimeError("BatchDecodeWithPagedKVCacheWrapper: begin_forward must come first")
         n_listed, nq, nkv, page, dtype = self._plan
+        # the reference's kernel reads the page count from the indptr given here; begin_forward has
+        # fixed it, so a different one is an error rather than a silently stale page count (a device
+        # tensor is not read back: that would stall the stream)
+        if (isinstance(paged_kv_indptr, torch.Tensor) and not paged_kv_indptr.is_cuda
+                and paged_kv_indptr.numel() == 2):
+            now = int(paged_kv_indptr.reshape(-1)[1]) - int(paged_kv_indptr.reshape(-1)[0])
+            if now != n_listed:
+                raise RuntimeError("paged_kv_indptr lists %d pages, begin_forward was given %d"
+                                   % (now, n_listed))
         _check_cuda_contig(q, "q", dtype, 3)
         _check_cuda_contig(o, "o", dtype, 3)
         _check_cuda_contig(paged_kv_data, "paged_kv_data", dtype, 5)

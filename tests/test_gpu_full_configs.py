@@ -176,6 +176,9 @@ def test_decode_wrapper_page_lists_against_oracle(gpu_device, layout, page_size,
         wrapper.forward(q.to(gpu_device), o, kv.to(gpu_device), idx.to(gpu_device),
                         torch.tensor([0, n_listed], dtype=torch.int32, device=gpu_device),
                         last_len, last_idx)
+    with pytest.raises(RuntimeError):   # a host indptr that disagrees with the plan of begin_forward
+        wrapper.forward(q.to(gpu_device), o, kv.to(gpu_device), idx.to(gpu_device),
+                        torch.tensor([0, n_listed + 1], dtype=torch.int32), last_len, last_idx)
     wrapper.end_forward()
     kvn = kv.numpy() if layout == "NHD" else kv.permute(0, 1, 3, 2, 4).numpy()   # [pool, 2, P, H, D]
     k_flat = kvn[:, 0].reshape(n_pool * page_size, H, D)

@@ -845,3 +845,31 @@ def test_paging_identity_vs_shuffled(gpu_device):
         outs.append((q_code.clone(), est.clone(), sel, o, o_f, sel_f))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+def test_split_merge_inside_the_launch_gives_the_same_bits_every_time(gpu_device):
+    """The attention over 1023 rows per head is cut into eight splits whose partial results are
+    merged by the last workgroup to arrive, inside the launch (write-through stores, an arrival
+    counter, cache-bypassing loads; csrc/split_merge.h).  A partial that is read before it has
+    arrived shows up as different output bits: 300 launches on changing inputs, each repeated, must
+    agree with themselves bit for bit, and the result must not depend on what the workspace held."""
+    L, budget = 9000, 1024
+    seq = _device_sequence(gpu_device, L, 99)
+    ctrl = T.make_controller(gpu_device, L, budget, 16, shuffle_seed=5)
+    T.fill_sequence(ctrl, seq.k[:L - 1], seq.v[:L - 1])
+    q_code = T.decode_append(ctrl, seq.q[None], seq.k[L - 1:], seq.v[L - 1:])
+    est = U.decode_estimate(q_code, ctrl, 0)
+    U.decode_topk(est, ctrl)
+    sel = ctrl.topk_dindices_buffer
+    g = torch.Generator(device=gpu_device).manual_seed(7)
+    for it in range(150):
+        q = (torch.randn(1, 32, 128, generator=g, device=gpu_device) * (1 + it % 5)).half()
+        a = U.decode_sparse_attn(q, ctrl, 0, sel).clone()
+        b = U.decode_sparse_attn(q, ctrl, 0, sel)
+        assert torch.equal(a, b), it
+    # the large-budget step merges its slabs the same way
+    for it in range(50):
+        q = (torch.randn(1, 32, 128, generator=g, device=gpu_device) * (1 + it % 3)).half()
+        a = U.decode_step(q, q_code, ctrl, 0).clone()
+        b = U.decode_step(q, q_code, ctrl, 0)
+        assert torch.equal(a, b), it
