@@ -152,6 +152,9 @@ def parse_args():
     ap.add_argument("--no-extra-legs", action="store_true",
                     help="headline workload only: skip the two extra timings of the step (caches built "
                          "with the other scale of the transform; a sequence of 33024 tokens)")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="headline workload only: skip the step timings of configs 1, 3 and 4 that ride "
+                         "in the same record")
     ap.add_argument("--no-e2e", action="store_true",
                     help="skip the end-to-end decode leg (random-init Llama-2-7B shape, 32768-token "
                          "prompt, 256 greedy tokens, sparse path against dense attention)")
@@ -330,7 +333,7 @@ def run_batched(args, w, lib, torch, U, _lib, dev):
     code_bytes = sum(L - 1 for L in lens) * H * 32
     step_bytes = sum(lens) * H * (D // 4) + B * 2 * budget * H * D * 2
     achieved = code_bytes / (cand_us * 1e-6) / 1e9
-    print(json.dumps({
+    return {
         "metric": "decode_attn_us_per_layer_batched_ragged", "value": round(step_us, 3), "unit": "us",
         "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(step_us / 1e3, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
@@ -351,7 +354,7 @@ def run_batched(args, w, lib, torch, U, _lib, dev):
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": code_bytes, "avg_launch_us": round(cand_us, 3)},
         "cpu_baseline": None,
-    }), flush=True)
+    }
 
 
 def main():
@@ -387,7 +390,8 @@ def main():
         import dataclasses
         w = dataclasses.replace(w, seq_lens=(args.kv_len,))
     if len(w.seq_lens) > 1:
-        return run_batched(args, w, lib, torch, U, _lib, dev)
+        print(json.dumps(run_batched(args, w, lib, torch, U, _lib, dev)), flush=True)
+        return
     result = run_single(args, w, lib, torch, U, _lib, dev, np, synth)
     if result is None:
         return
@@ -773,6 +777,32 @@ def run_single(args, w, lib, torch, U, _lib, dev, np, synth):
         "cpu_baseline": cpu,
     }
     result.update(extra_legs)
+    # ---- the other kernel workloads of the benchmark definition, same protocol, in the same record --
+    # (configs 1, 3 and 4: the step and its two kernels; the full record of each is what
+    # `bench.py --workload <name>` prints)
+    if extra_legs and not args.no_other_workloads:
+        others = {}
+        # 4 layer caches for the long sequence: 128K tokens x 4 layers = 8.6 GB
+        few = argparse.Namespace(**{**vars(args), "layers": min(args.layers, 4)})
+        for name in ("c1_4k_b64", "c4_128k_b256"):
+            w2 = synth.WORKLOADS[name]
+            leg = time_step_leg(few if name.startswith("c4") else args, w2, w2.seq_lens[0],
+                                args.hadamard_scale, lib, torch, U, _lib, dev, np, synth, flush)
+            bytes2 = w2.seq_lens[0] * H * (D // 4) + 2 * w2.budget * H * D * 2
+            leg["token_budget"] = w2.budget
+            leg["algorithmic_bytes_per_step"] = bytes2
+            leg["frac_of_hbm_roofline"] = round(bytes2 / (leg["value"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+            others[name] = leg
+            log(f"{name}: step {leg['value']:.2f} us (estimate+select {leg.get('estimate_select')}, "
+                f"select+attend {leg.get('select_attend')})")
+        rb = run_batched(args, synth.WORKLOADS["c3_ragged16_b128"], lib, torch, U, _lib, dev)
+        others["c3_ragged16_b128"] = {k: rb[k] for k in ("value", "unit", "step_kernels_us",
+                                                           "frac_of_hbm_roofline",
+                                                           "algorithmic_bytes_per_step")}
+        others["c3_ragged16_b128"]["seq_lens"] = rb["config"]["seq_lens"]
+        others["c3_ragged16_b128"]["estimator_frac_of_hbm_roofline"] = rb["roofline"]["frac"]
+        log(f"c3_ragged16_b128: step {rb['value']:.2f} us {rb['step_kernels_us']}")
+        result["other_workloads"] = others
     return result
 
 
