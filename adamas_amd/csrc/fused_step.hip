@@ -429,8 +429,8 @@ struct SelectAttendShared {
   alignas(16) float qkv_now[3][kHeadDim];
 };
 
-// Two candidate slots per thread: slots 2*tid and 2*tid + 1 of the head's n_chunks * kc slots (at
-// most kStepMaxSlots; both belong to one chunk since kc is even).
+// kSlots (2 or 4) candidate slots per thread: slots kSlots*tid .. of the head's n_chunks * kc slots
+// (at most kSlots * 512; they belong to one chunk since kc is a multiple of 8).
 // q_code [sequence*heads][16], code_data: the query codes and the code cache the first launch worked
 // with, read only when a chunk has to be scored again; dist_scratch [sequence*heads][dist_stride]
 // u16 then holds that chunk's distances (rows are private to a workgroup).
@@ -438,7 +438,7 @@ struct SelectAttendShared {
 // embedding to the query and to the new key itself, appends the new key, its code and the new value
 // (the workgroup of the first query head of a key/value head), and attends the current token from
 // registers instead of reading it back: the decode append needs no launch of its own.
-template <bool kBf16, bool kHnd, bool kFromQkv = false>
+template <int kSlots, bool kBf16, bool kHnd, bool kFromQkv = false>
 __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     const __half* __restrict__ q, const __half* __restrict__ kv_data,
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
@@ -450,7 +450,8 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     uint16_t* __restrict__ dist_scratch, int64_t dist_stride, QkvSource src = QkvSource(),
     __half* kv_append = nullptr, uint16_t* code_append = nullptr) {
   static_assert(kAttThreads == kHistBins, "one thread per distance value");
-  static_assert(kStepMaxSlots == 2 * kAttThreads, "two candidate slots per thread");
+  static_assert(kSlots == 2 || kSlots == 4, "one or two 128-bit loads of candidates per thread");
+  static_assert(kStepMaxSlots == 4 * kAttThreads, "at most four candidate slots per thread");
   static_assert(kStepMaxChunks == kWave, "the flags of all chunks fit one ballot");
   __shared__ SelectAttendShared sh;
   const uint32_t head = blockIdx.x;
@@ -465,10 +466,14 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   // ---- the candidates of this head: two slots per thread --------------------------------------------
   // (asked for ahead of everything that waits for the sequence length: the list of a sequence
   // without tokens is valid memory, if meaningless)
-  const uint32_t slot0 = 2u * tid;
+  const uint32_t slot0 = static_cast<uint32_t>(kSlots) * tid;
   const bool have = slot0 < n_slots;
-  uint4 raw = make_uint4(~0u, ~0u, ~0u, ~0u);  // an unused slot is all ones
-  if (have) raw = *reinterpret_cast<const uint4*>(crow + slot0);  // lists are 64-byte aligned
+  uint4 raw[kSlots / 2];
+#pragma unroll
+  for (int j = 0; j < kSlots / 2; ++j) {
+    raw[j] = make_uint4(~0u, ~0u, ~0u, ~0u);  // an unused slot is all ones
+    if (have) raw[j] = *reinterpret_cast<const uint4*>(crow + slot0 + 2 * j);  // lists are 64-byte aligned
+  }
 
   // K row of the current token: a chain of three dependent scalar loads, started early so that it
   // has long finished when the row list is closed
@@ -521,14 +526,21 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   }
 
   // a candidate is (distance << 48) | (token offset in its chunk << 32) | K row index
-  uint32_t key[2] = {raw.y >> 16, raw.w >> 16};  // an unused slot reads 0xffff: above every threshold
-  const uint32_t off[2] = {raw.y & 0xffffu, raw.w & 0xffffu};
-  const uint32_t krow[2] = {raw.x, raw.z};
+  uint32_t key[kSlots], off[kSlots], krow[kSlots];
+#pragma unroll
+  for (int j = 0; j < kSlots / 2; ++j) {
+    key[2 * j] = raw[j].y >> 16;  // an unused slot reads 0xffff: above every threshold
+    key[2 * j + 1] = raw[j].w >> 16;
+    off[2 * j] = raw[j].y & 0xffffu;
+    off[2 * j + 1] = raw[j].w & 0xffffu;
+    krow[2 * j] = raw[j].x;
+    krow[2 * j + 1] = raw[j].z;
+  }
   const uint32_t chunk_mine = slot0 >> geom.kc_log2;
   const uint32_t chunk_tok0 = chunk_first_unit(geom, chunk_mine) * kStepUnit;
   __syncthreads();  // the histogram is cleared
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < kSlots; ++i)
     if (key[i] < static_cast<uint32_t>(kHistBins)) atomicAdd(&sh.hist[key[i]], 1u);
   if (kFromQkv && wave < 3) {
     float x0, x1;
@@ -554,8 +566,10 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   // come before them in slot order (wave prefix scan + the totals of the earlier waves).
   uint32_t rb, re, list_below;
   auto rank_slots = [&]() __attribute__((always_inline)) {
-    const uint32_t mine = (key[0] < plan.thr ? 1u : 0u) + (key[1] < plan.thr ? 1u : 0u) +
-                          (((key[0] == plan.thr ? 1u : 0u) + (key[1] == plan.thr ? 1u : 0u)) << 16);
+    uint32_t mine = 0;
+#pragma unroll
+    for (int i = 0; i < kSlots; ++i)
+      mine += (key[i] < plan.thr ? 1u : 0u) + ((key[i] == plan.thr ? 1u : 0u) << 16);
     const uint32_t incl = wave_inclusive_scan_dpp(mine);
     if (lane == kWave - 1) sh.wclass[wave] = incl;
     __syncthreads();
@@ -563,7 +577,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     const uint4 lo = *reinterpret_cast<const uint4*>(&sh.wclass[0]);
     const uint4 hi = *reinterpret_cast<const uint4*>(&sh.wclass[4]);
     const uint32_t t[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    uint32_t before = 0, all = 0;  // the 16-bit fields cannot carry: at most 1024 slots
+    uint32_t before = 0, all = 0;  // the 16-bit fields cannot carry: at most 2048 slots
 #pragma unroll
     for (int w = 0; w < 8; ++w) {
       before += w < wave ? t[w] : 0u;
@@ -576,12 +590,12 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
   };
   const bool want_pos = sel_out != nullptr;
   // writes the selected ones of this thread's slots into the row list; `tie_shift` tied tokens of
-  // re-scored chunks come before this thread's chunk.  Returns whether the second slot was selected.
+  // re-scored chunks come before this thread's chunk.  Returns whether the last slot was selected.
   auto emit_slots = [&](uint32_t tie_shift) __attribute__((always_inline)) -> bool {
     uint32_t pb = rb, pe = re + tie_shift;
     bool last_selected = false;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kSlots; ++i) {
       const bool is_b = key[i] < plan.thr, is_e = key[i] == plan.thr;
       const bool take = is_b || (is_e && pe < plan.quota);
       if (take) {
@@ -601,7 +615,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     // The list of a chunk is a prefix of the chunk in (distance, index) order.  If its last entry is
     // selected and the chunk holds more tokens than the list, tokens outside the list may belong to
     // the selection too: the chunk is scored again below.
-    if (last_selected && ((slot0 + 1u) & (geom.kc - 1u)) == geom.kc - 1u) {
+    if (last_selected && ((slot0 + kSlots - 1u) & (geom.kc - 1u)) == geom.kc - 1u) {
       const uint32_t chunk_len = min(chunk_units(geom, chunk_mine) * kStepUnit, n - chunk_tok0);
       if (chunk_len > geom.kc) {
         sh.flag[chunk_mine] = 1u;
@@ -619,7 +633,7 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
     const bool mine_flagged = have && ((fmask >> chunk_mine) & 1ull) != 0;
     if (mine_flagged) {  // the listed entries of such a chunk leave the count: its tokens come back below
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < kSlots; ++i) {
         if (key[i] < static_cast<uint32_t>(kHistBins)) atomicSub(&sh.hist[key[i]], 1u);
         key[i] = 0xffffu;
       }
@@ -1227,8 +1241,8 @@ static int step_attend_impl(const void* q, void* kv_data, void* code_data,
   if (!fused_eligible(w)) return ADAMAS_E_UNSUPPORTED;
   char* ws = static_cast<char*>(workspace);
   const StepPlan& plan = w.plan;
-#define ADAMAS_LAUNCH_SELATT_BF(BF, HND, FROMQKV)                                                \
-  hipLaunchKernelGGL((select_attend_kernel<BF, HND, FROMQKV>), dim3(num_heads, batch),           \
+#define ADAMAS_LAUNCH_SELATT_S(SLOTS, BF, HND, FROMQKV)                                          \
+  hipLaunchKernelGGL((select_attend_kernel<SLOTS, BF, HND, FROMQKV>), dim3(num_heads, batch),    \
                      dim3(kAttThreads), 0,                                                       \
                      static_cast<hipStream_t>(stream), static_cast<const __half*>(q),           \
                      static_cast<const __half*>(kv_data), page_indices, page_indptr, seq_lens,  \
@@ -1242,6 +1256,12 @@ static int step_attend_impl(const void* q, void* kv_data, void* code_data,
                      reinterpret_cast<uint16_t*>(ws + w.dist_off), w.dist_stride,               \
                      qsrc ? *qsrc : QkvSource(), static_cast<__half*>(kv_data),                 \
                      static_cast<uint16_t*>(code_data))
+#define ADAMAS_LAUNCH_SELATT_BF(BF, HND, FROMQKV)     \
+  if (plan.chunks * plan.kc > 2 * kAttThreads) {      \
+    ADAMAS_LAUNCH_SELATT_S(4, BF, HND, FROMQKV);      \
+  } else {                                            \
+    ADAMAS_LAUNCH_SELATT_S(2, BF, HND, FROMQKV);      \
+  }
 #define ADAMAS_LAUNCH_SELATT(FROMQKV)                 \
   if (bf16 && hnd) {                                  \
     ADAMAS_LAUNCH_SELATT_BF(true, true, FROMQKV);     \
@@ -1259,6 +1279,7 @@ static int step_attend_impl(const void* q, void* kv_data, void* code_data,
   }
 #undef ADAMAS_LAUNCH_SELATT
 #undef ADAMAS_LAUNCH_SELATT_BF
+#undef ADAMAS_LAUNCH_SELATT_S
   ADAMAS_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

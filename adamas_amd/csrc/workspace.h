@@ -18,7 +18,7 @@ constexpr uint32_t kFusedMaxPasses = 4;              // a workgroup covers at mo
 constexpr uint32_t kFusedMaxSel = 255;               // largest budget-1 of the two-launch path
 constexpr uint32_t kStepUnit = 16;                   // chunk boundaries are multiples of 16 tokens
 constexpr uint32_t kStepMaxChunks = 64;              // token chunks per sequence of the two-launch step
-constexpr uint32_t kStepMaxSlots = 1024;             // candidate slots per head: chunks x slots per chunk
+constexpr uint32_t kStepMaxSlots = 2048;             // candidate slots per head: chunks x slots per chunk
 constexpr uint32_t kStepWorkgroups = 256;            // the estimator aims at one workgroup per CU of an MI355X
 
 // Geometry of the two-launch step (estimate_select_kernel, select_attend_kernel), fixed on the host
@@ -107,8 +107,12 @@ inline StepPlan step_plan(uint32_t batch, uint32_t num_heads, uint32_t max_seq_l
   if (p.passes == 0 || p.passes > kFusedMaxPasses) return p;
   p.partial = (p.units_r != 0 || p.units_q % pass_units != 0) ? 1u : 0u;
   // slots per chunk: the whole budget where the lists of all chunks fit, else what fits (at least
-  // 16: the second launch re-scores the rare chunk that holds more of the selection than its list)
-  const uint32_t fit = pow2_floor(kStepMaxSlots / p.chunks);
+  // 16: the second launch re-scores the rare chunk that holds more of the selection than its list).
+  // One sequence: 1024 slots per head (two per thread of the second launch; a chunk holds
+  // budget / chunks of the selection on average, a small fraction of its list).  Several sequences:
+  // the chunks are sized for the longest one, a short sequence spreads its selection over few of
+  // them, and twice the slots keep those lists from running out.
+  const uint32_t fit = pow2_floor((batch == 1 ? kStepMaxSlots / 2 : kStepMaxSlots) / p.chunks);
   p.kc = std::max(8u, std::min(fit, pow2_ceil(budget - 1)));
   p.kc_log2 = 0;
   while ((1u << p.kc_log2) < p.kc) ++p.kc_log2;
