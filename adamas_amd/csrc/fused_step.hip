@@ -810,24 +810,38 @@ __global__ __launch_bounds__(kAttThreads) void select_attend_kernel(
 // through memory and the wait for it.
 constexpr int kHsaThreads = 256;
 constexpr int kHsaWaves = kHsaThreads / kWave;
-constexpr int kHsaItems = 16;                                    // distances per thread
-constexpr uint32_t kHsaSlab = kHsaThreads * kHsaItems;           // 4096 tokens per workgroup
-constexpr uint32_t kHsaSlabChunks = kHsaSlab / kFusedBlock;      // 8 histogram rows per slab
+constexpr int kHsaMaxItems = 16;                                 // distances per thread, at most
+constexpr uint32_t kHsaMaxSlab = kHsaThreads * kHsaMaxItems;     // 4096 tokens per workgroup, at most
 constexpr int kHsaGroups = kHsaThreads / 16;
-constexpr uint32_t kHsaMaxTokens = kHsaSlab * 32;                // 32 slabs per head at most
+constexpr uint32_t kHsaMaxTokens = kHsaMaxSlab * 32;             // 32 slabs per head at most
 
+// Tokens per thread of hist_select_attend_kernel (4, 8 or 16: slabs of 1024, 2048 or 4096 tokens).
+// One CU gathers scattered rows slowly, so a slab should not hold much more than 256 selected rows:
+// the slab is halved while that leaves at most max(slabs of 4096 tokens, min(16, budget / 256))
+// slabs per head (up to 16 slabs the merge inside the launch stays cheap).
+inline int hsa_items(uint32_t max_seq_len, uint32_t budget) {
+  const uint32_t n = max_seq_len > 1 ? max_seq_len - 1 : 1;
+  const uint32_t most =
+      std::max((n + kHsaMaxSlab - 1) / kHsaMaxSlab, std::min(16u, (budget + 255u) / 256u));
+  int items = kHsaMaxItems;
+  while (items > 4 && (n + kHsaThreads * (items / 2) - 1) / (kHsaThreads * (items / 2)) <= most)
+    items /= 2;
+  return items;
+}
+
+template <int kItems>
 struct HistSelectAttendShared {
   alignas(16) uint32_t all[kHsaWaves][kHistBins];  // partial sums over all chunk rows
   alignas(16) uint32_t pre[kHsaWaves][kHistBins];  // partial sums over the chunk rows before the slab
   uint32_t wtot[kHsaWaves], wpre[kHsaWaves], wclass[kHsaWaves];
   uint32_t pre_tied;   // tokens at the threshold distance in the chunks before the slab
   SelectPlan plan;
-  int32_t rows[kHsaSlab + 1];  // K rows of the slab's selected tokens (slab 0: then the current token)
+  int32_t rows[kHsaThreads * kItems + 1];  // K rows of the slab's selected tokens (slab 0: then the current token)
   MergeShared<kHsaGroups> merge;
   uint32_t is_last;
 };
 
-template <bool kBf16, bool kHnd>
+template <bool kBf16, bool kHnd, int kItems>
 __global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
     const __half* __restrict__ q, const __half* __restrict__ kv_data,
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
@@ -837,7 +851,10 @@ __global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
     uint32_t* __restrict__ counters, uint32_t num_heads, uint32_t num_kv_heads, uint32_t kv_inv16,
     uint32_t page_size, float scale_log2) {
   static_assert(kHsaThreads * 2 == kHistBins, "two bins per thread in the prefix sum");
-  __shared__ HistSelectAttendShared sh;
+  static_assert(kItems == 4 || kItems == 8 || kItems == 16, "whole histogram rows per slab");
+  constexpr uint32_t kSlab = kHsaThreads * kItems;         // tokens per workgroup
+  constexpr uint32_t kSlabChunks = kSlab / kFusedBlock;    // histogram rows per slab
+  __shared__ HistSelectAttendShared<kItems> sh;
   const uint32_t bh = blockIdx.x, slab = blockIdx.y;
   const uint32_t b = bh / num_heads, head = bh - b * num_heads;
   const uint32_t tid = threadIdx.x;
@@ -855,36 +872,44 @@ __global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
     return;
   }
   const uint32_t n = static_cast<uint32_t>(seq_len) - 1u;                 // past tokens
-  const uint32_t n_split = n ? (n + kHsaSlab - 1) / kHsaSlab : 1u;        // slabs that hold tokens
+  const uint32_t n_split = n ? (n + kSlab - 1) / kSlab : 1u;              // slabs that hold tokens
   if (slab >= n_split) return;
-  const uint32_t slab_base = slab * kHsaSlab;
-  // thread t holds the 16 consecutive tokens t*16 .. t*16+15 of the slab: distances and K rows,
+  const uint32_t slab_base = slab * kSlab;
+  // thread t holds the kItems consecutive tokens t*kItems .. of the slab: distances and K rows,
   // asked for first
-  const uint32_t e0 = slab_base + tid * kHsaItems;
-  uint32_t keys[kHsaItems], trow[kHsaItems];
+  const uint32_t e0 = slab_base + tid * kItems;
+  uint32_t keys[kItems], trow[kItems];
   {
-    const uint16_t* vrow = dist + static_cast<int64_t>(bh) * dist_stride + e0;  // 16-byte aligned
+    const uint16_t* vrow = dist + static_cast<int64_t>(bh) * dist_stride + e0;  // 2*kItems-byte aligned
     const uint32_t* rm = rowmap + static_cast<int64_t>(b) * dist_stride + e0;
-    uint4 kraw[2], rraw[4];
+    uint32_t kw[kItems / 2];  // two distances per word
+    uint4 rraw[kItems / 4];
+    if (kItems == 4) {
+      const uint2 v = e0 < n ? *reinterpret_cast<const uint2*>(vrow) : make_uint2(~0u, ~0u);
+      kw[0] = v.x;
+      kw[1] = v.y;
+    } else {
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
-      kraw[j] = e0 + 8 * j < n ? *reinterpret_cast<const uint4*>(vrow + 8 * j)
-                               : make_uint4(~0u, ~0u, ~0u, ~0u);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      rraw[j] = e0 + 4 * j < n ? *reinterpret_cast<const uint4*>(rm + 4 * j)
-                               : make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const uint32_t w[4] = {kraw[j].x, kraw[j].y, kraw[j].z, kraw[j].w};
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const uint32_t v = (w[i >> 1] >> (16 * (i & 1))) & 0xffffu;
-        keys[8 * j + i] = e0 + 8 * j + i < n ? v : 0xffffu;  // past the end: above every threshold
+      for (int j = 0; j < kItems / 8; ++j) {
+        const uint4 v = e0 + 8 * j < n ? *reinterpret_cast<const uint4*>(vrow + 8 * j)
+                                       : make_uint4(~0u, ~0u, ~0u, ~0u);
+        kw[4 * j] = v.x;
+        kw[4 * j + 1] = v.y;
+        kw[4 * j + 2] = v.z;
+        kw[4 * j + 3] = v.w;
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kItems / 4; ++j)
+      rraw[j] = e0 + 4 * j < n ? *reinterpret_cast<const uint4*>(rm + 4 * j)
+                               : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) {
+      const uint32_t v = (kw[i >> 1] >> (16 * (i & 1))) & 0xffffu;
+      keys[i] = e0 + i < n ? v : 0xffffu;  // past the end: above every threshold
+    }
+#pragma unroll
+    for (int j = 0; j < kItems / 4; ++j) {
       trow[4 * j] = rraw[j].x;
       trow[4 * j + 1] = rraw[j].y;
       trow[4 * j + 2] = rraw[j].z;
@@ -904,7 +929,7 @@ __global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
   // ---- chunk rows (16-bit counts): thread (part, seg) adds bins 8*seg .. 8*seg+7 of rows part, part+4, ...
   {
     const uint32_t part = tid >> 6, seg = tid & 63u;
-    const uint32_t c_first = slab * kHsaSlabChunks;  // chunks below it precede the slab
+    const uint32_t c_first = slab * kSlabChunks;  // chunks below it precede the slab
     const unsigned char* hb = reinterpret_cast<const unsigned char*>(hist) +
                               static_cast<size_t>(bh) * n_chunks * (2 * kHistBins) + seg * 16u;
     const uint32_t rows_used = min(n_chunks, (n + kFusedBlock - 1) / kFusedBlock);  // rows of this sequence
@@ -984,10 +1009,10 @@ __global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
   // ---- selected tokens before the slab, class masks and ranks inside it
   const uint32_t mine_pre = (2 * tid < plan.thr ? cp0 : 0u) + (2 * tid + 1 < plan.thr ? cp1 : 0u);
   const uint32_t wave_pre = wave_sum(mine_pre);
-  uint32_t below[kHsaItems / 4], equal[kHsaItems / 4];
-  raw_class_masks<kHsaItems>(keys, plan.thr, below, equal);
+  uint32_t below[kItems / 4], equal[kItems / 4];
+  raw_class_masks<kItems>(keys, plan.thr, below, equal);
   uint32_t total;
-  const uint32_t excl = lane_scan<kHsaItems / 4>(below, equal, total);  // below | tied << 16
+  const uint32_t excl = lane_scan<kItems / 4>(below, equal, total);  // below | tied << 16
   if (lane == 0) {
     sh.wpre[wave] = wave_pre;
     sh.wclass[wave] = total;
@@ -1006,7 +1031,7 @@ __global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
   const uint32_t tied_left = plan.quota > pre_tied ? plan.quota - pre_tied : 0u;
   const uint32_t slab_tied_taken = min(slab_tied, tied_left);
   // positions in the whole selection: the tokens below the threshold in index order, then the ties
-  lane_emit<kHsaItems / 4>(below, equal, plan.n_below, plan.quota,
+  lane_emit<kItems / 4>(below, equal, plan.n_below, plan.quota,
                            base_b + (before & 0xffffu) + (excl & 0xffffu),
                            pre_tied + (before >> 16) + (excl >> 16),
                            [&](uint32_t pos, int i) __attribute__((always_inline)) {
@@ -1209,7 +1234,7 @@ extern "C" int adamas_step_candidates(const void* q_code, const void* code_data,
                                   page_size, max_seq_len, page_table_stride, 0u, stream);
 }
 
-// qsrc != nullptr (fp16, NHD): q is made in the kernel from the fused projection, the new token is
+// qsrc != nullptr: q is made in the kernel from the fused projection, the new token is
 // appended by it (kv_data and code_data are written)
 static int step_attend_impl(const void* q, void* kv_data, void* code_data,
                             const int32_t* page_indices,
@@ -1401,9 +1426,11 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
     // selection from the histograms and attention over the selected rows, one launch
     const bool bf16 = (flags & ADAMAS_F_BF16) != 0, hnd = (flags & ADAMAS_F_HND) != 0;
-    const dim3 hgrid(batch * num_heads, (max_seq_len - 1 + kHsaSlab - 1) / kHsaSlab);
-#define ADAMAS_LAUNCH_HSA(BF, HND)                                                                 \
-  hipLaunchKernelGGL((hist_select_attend_kernel<BF, HND>), hgrid, dim3(kHsaThreads), 0, s,         \
+    const int items = hsa_items(max_seq_len, budget);
+    const uint32_t slab_tokens = kHsaThreads * static_cast<uint32_t>(items);
+    const dim3 hgrid(batch * num_heads, (max_seq_len - 1 + slab_tokens - 1) / slab_tokens);
+#define ADAMAS_LAUNCH_HSA_I(BF, HND, ITEMS)                                                        \
+  hipLaunchKernelGGL((hist_select_attend_kernel<BF, HND, ITEMS>), hgrid, dim3(kHsaThreads), 0, s,  \
                      static_cast<const __half*>(q), static_cast<const __half*>(kv_data),           \
                      page_indices, page_indptr, seq_lens, dist, w.dist_stride,                     \
                      reinterpret_cast<const uint16_t*>(hist), w.hist_stride, rowmap, n_sel,        \
@@ -1412,6 +1439,14 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
                      reinterpret_cast<uint32_t*>(ws + w.counters_off), num_heads, num_kv_heads,    \
                      group_inv16(num_heads / num_kv_heads), page_size,                             \
                      sm_scale * 1.4426950408889634f)
+#define ADAMAS_LAUNCH_HSA(BF, HND)          \
+  if (items == 4) {                         \
+    ADAMAS_LAUNCH_HSA_I(BF, HND, 4);        \
+  } else if (items == 8) {                  \
+    ADAMAS_LAUNCH_HSA_I(BF, HND, 8);        \
+  } else {                                  \
+    ADAMAS_LAUNCH_HSA_I(BF, HND, 16);       \
+  }
     if (bf16 && hnd) {
       ADAMAS_LAUNCH_HSA(true, true);
     } else if (bf16) {
@@ -1422,6 +1457,7 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
       ADAMAS_LAUNCH_HSA(false, false);
     }
 #undef ADAMAS_LAUNCH_HSA
+#undef ADAMAS_LAUNCH_HSA_I
     ADAMAS_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }

@@ -550,7 +550,7 @@ def test_step_truncated_chunk_lists_are_rescored(gpu_device, kv_len, budget, pag
 @pytest.mark.timeout(900)
 @pytest.mark.parametrize("kv_len,budget,page_size", [
     (5000, 300, 16), (20000, 512, 16), (32768, 1024, 16), (9000, 4096, 3), (40000, 2048, 1),
-    (2000, 257, 16), (131072, 700, 16),
+    (2000, 257, 16), (131072, 700, 16), (16384, 2048, 16), (8192, 4096, 16),
 ])
 def test_step_large_budgets(gpu_device, kv_len, budget, page_size):
     """Budgets above 256 (the reference's kernel benchmarks go up to 4096): the step runs as
