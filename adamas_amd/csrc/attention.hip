@@ -13,14 +13,17 @@
 
 namespace adamas {
 
-constexpr int kTile = 8;             // rows per group per tile
-// A workgroup has 256 or 512 threads = 16 or 32 groups, i.e. 128 or 256 rows per tile.  Lists of up to
-// 1024 rows are cut into splits of 128 rows (up to 8 per head: enough workgroups to fill the chip).
-// Longer lists take the wide workgroup and splits of 256 rows: as many rows in flight per CU, half as
-// many partial results to merge, so that up to 4096 rows the merge stays inside the launch.
-// (Not splitting at all is far slower: one 1024-thread workgroup per head gathers 1024 rows in 25 us
-// against 13 us for eight splits - a single CU pulls scattered rows at a few tens of GB/s.)
-constexpr uint32_t kWideRowsFrom = 1025;
+constexpr int kTile = 8;             // rows per group per tile, at most
+// A workgroup has 256 or 512 threads = 16 or 32 groups of 16 lanes; a group has 2, 4 or 8 rows in
+// flight, and a split is one such round of loads.  One CU gathers scattered rows slowly (a single
+// 1024-thread workgroup per head takes 25 us for 1024 rows, eight splits 13 us), a group finishes
+// sooner the fewer rows it has to ask for, and publishing a partial result costs about a
+// microsecond.  Hence: 32 groups from 65 rows on; up to 128 rows one split (4 rows per group, no
+// merge); up to 512 rows splits of 64 rows (2 per group, at most 8 splits); up to 2048 rows splits
+// of 128 (at most 16); beyond that splits of 256.  Measured at 32 heads, rows = 128 / 256 / 512 /
+// 1024 / 2048 / 4096, in us: 5.8 / 6.5 / 7.4 / 9.7 / 14.2 / 20.6 (with 16 groups of 8 rows and splits
+// of 128 rows up to 1024 rows, 256 beyond: 7.5 / 9.5 / 10.1 / 12.4 / 15.8 / 20.6).
+constexpr uint32_t kWideRowsFrom = 65;
 constexpr uint32_t kDeferredMergeSplits = 24;  // splits from which the partials get a merge launch
 // (measured at 32768 tokens, 32 heads: 16 splits 14.7 us merged inside the launch, 15.8 us with a merge
 // launch; 32 splits 26.6 against 22.5 us)
@@ -31,7 +34,7 @@ struct AttnShared {
   uint32_t is_last;
 };
 
-template <bool kBf16, bool kHnd, int kThreads = 256>
+template <bool kBf16, bool kHnd, int kThreads = 256, int kTileRows = kTile>
 __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
     const __half* __restrict__ q, const __half* __restrict__ kv_data,
     const int32_t* __restrict__ page_indices, const int32_t* __restrict__ page_indptr,
@@ -68,7 +71,7 @@ __global__ __launch_bounds__(kThreads) void sparse_decode_kernel(
   SoftmaxState st;
   // (token positions through the page table: branching around unused entries measured faster
   // here than loading always, 7.9 against 8.0 us at 128 rows)
-  attend_rows<kGroups, kTile, false, kBf16>(kv, qf, g, row_begin, row_end,
+  attend_rows<kGroups, kTileRows, false, kBf16>(kv, qf, g, row_begin, row_end,
                               [&](uint32_t r) __attribute__((always_inline)) -> int32_t {
                                 if (dense) return static_cast<int32_t>(r);
                                 return (r < n_sel) ? sel[r] : seq_len - 1;
@@ -878,10 +881,11 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
     return merge_launch();
   }
   const uint32_t n_rows = sel_idx ? n_sel + 1u : max_seq_len;
-  // one tile of rows per split (128, or 256 with the wide workgroup), more where that would take
-  // more than kMaxSplits splits
+  // one round of loads per split (see the rule at kWideRowsFrom; up to 128 rows that is a single
+  // split, which needs no workspace), more where that would take more than kMaxSplits splits
   const bool wide = n_rows >= kWideRowsFrom;
-  const uint32_t rows_per_iter = (wide ? 32u : 16u) * kTile;
+  const uint32_t tile = n_rows <= 128 ? 4u : n_rows <= 512 ? 2u : n_rows <= 2048 ? 4u : 8u;
+  const uint32_t rows_per_iter = (wide ? 32u : 16u) * tile;
   uint32_t rows_per_split = rows_per_iter;
   uint32_t n_split = (n_rows + rows_per_split - 1) / rows_per_split;
   if (n_split > kMaxSplits) {
@@ -900,18 +904,22 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
   }
   // from kDeferredMergeSplits splits on, the merge is a second short launch
   const uint32_t deferred = n_split >= kDeferredMergeSplits ? 1u : 0u;
-#define ADAMAS_LAUNCH_SPARSE_T(BF, HND, T)                                                       \
-  hipLaunchKernelGGL((sparse_decode_kernel<BF, HND, T>), dim3(n_split, num_heads, batch),        \
+#define ADAMAS_LAUNCH_SPARSE_T(BF, HND, T, TILE)                                                 \
+  hipLaunchKernelGGL((sparse_decode_kernel<BF, HND, T, TILE>), dim3(n_split, num_heads, batch),  \
                      dim3(T), 0, static_cast<hipStream_t>(stream),                               \
                      static_cast<const __half*>(q), static_cast<const __half*>(kv_data),         \
                      page_indices, page_indptr, seq_lens, sel_idx, sel_stride, n_sel,            \
                      static_cast<__half*>(out), partial, counters, num_heads, num_kv_heads,      \
                      page_size, scale_log2, rows_per_split, deferred)
-#define ADAMAS_LAUNCH_SPARSE_L(BF, HND)       \
-  if (wide) {                                 \
-    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512);     \
-  } else {                                    \
-    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 256);     \
+#define ADAMAS_LAUNCH_SPARSE_L(BF, HND)          \
+  if (!wide) {                                   \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 256, 4);     \
+  } else if (tile == 2) {                        \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512, 2);     \
+  } else if (tile == 4) {                        \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512, 4);     \
+  } else {                                       \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512, 8);     \
   }
 #define ADAMAS_LAUNCH_SPARSE(BF)        \
   if (flags & ADAMAS_F_HND) {           \

@@ -816,13 +816,16 @@ constexpr int kHsaGroups = kHsaThreads / 16;
 constexpr uint32_t kHsaMaxTokens = kHsaMaxSlab * 32;             // 32 slabs per head at most
 
 // Tokens per thread of hist_select_attend_kernel (4, 8 or 16: slabs of 1024, 2048 or 4096 tokens).
-// One CU gathers scattered rows slowly, so a slab should not hold much more than 256 selected rows:
-// the slab is halved while that leaves at most max(slabs of 4096 tokens, min(16, budget / 256))
-// slabs per head (up to 16 slabs the merge inside the launch stays cheap).
+// One CU gathers scattered rows slowly, so the slab is halved while that leaves at most
+// max(slabs of 4096 tokens, min(16, budget / 64)) slabs per head: about 64 selected rows per
+// workgroup where the length allows it, and never more than 16 slabs for the sake of the rows
+// (beyond that the merge inside the launch costs more than the shorter gather saves).  Measured
+// against slabs of 4096 tokens throughout: 8192 tokens, budget 4096: 41.0 -> 24.8 us; 16384 / 1024:
+// 20.1 -> 18.4; 32768 / 1024: 23.3 -> 22.7; a target of 32 rows or a cap of 32 slabs is slower.
 inline int hsa_items(uint32_t max_seq_len, uint32_t budget) {
   const uint32_t n = max_seq_len > 1 ? max_seq_len - 1 : 1;
   const uint32_t most =
-      std::max((n + kHsaMaxSlab - 1) / kHsaMaxSlab, std::min(16u, (budget + 255u) / 256u));
+      std::max((n + kHsaMaxSlab - 1) / kHsaMaxSlab, std::min(16u, (budget + 63u) / 64u));
   int items = kHsaMaxItems;
   while (items > 4 && (n + kHsaThreads * (items / 2) - 1) / (kHsaThreads * (items / 2)) <= most)
     items /= 2;
@@ -1057,9 +1060,15 @@ __global__ __launch_bounds__(kHsaThreads) void hist_select_attend_kernel(
   set_kv_layout_static<kHnd>(kv, kv_head_of(head, kv_inv16), c16, num_kv_heads, page_size);
   kv.seq_len = seq_len;
   SoftmaxState st;
-  attend_rows<kHsaGroups, 8, true, kBf16, true>(
-      kv, qf, g, 0u, n_rows,
-      [&](uint32_t r) __attribute__((always_inline)) -> int32_t { return sh.rows[r]; }, st);
+  // (a group asks for 2, 4 or 8 rows at a time: slots past the end load the last row again, so the
+  // round is no larger than the slab's rows need)
+  auto row_of = [&](uint32_t r) __attribute__((always_inline)) -> int32_t { return sh.rows[r]; };
+  if (n_rows <= kHsaGroups * 2u)
+    attend_rows<kHsaGroups, 2, true, kBf16, true>(kv, qf, g, 0u, n_rows, row_of, st);
+  else if (n_rows <= kHsaGroups * 4u)
+    attend_rows<kHsaGroups, 4, true, kBf16, true>(kv, qf, g, 0u, n_rows, row_of, st);
+  else
+    attend_rows<kHsaGroups, 8, true, kBf16, true>(kv, qf, g, 0u, n_rows, row_of, st);
   float M, L, O;
   merge_groups<kHsaGroups>(st, g, c16, tid, sh.merge, M, L, O);
   if (n_split == 1) {
