@@ -1,12 +1,12 @@
 // Paged decode attention over a per-head list of token positions (gfx950).
 //
-// grid = (splits, heads, batch), 256 threads = 16 groups of 16 lanes.  A K or V row of one head is
-// 128 fp16 = 256 bytes = 16 lanes x 128-bit, so a group owns a row and a lane owns 8 channels.
-// Each group walks its rows in tiles of 8: 8 K loads and 8 V loads are issued before any of them is
-// used, the dot products are reduced over the 16 lanes, and an fp32 online softmax (base 2) keeps
-// (m, l, o[8]) per lane.  Groups are merged through LDS; when a head is cut into several splits the
-// partial (m, l, o[128]) go to the workspace and the last workgroup to arrive for that head merges
-// them, so there is no second launch.
+// grid = (splits, heads, batch), 256 - 1024 threads = 16 - 64 groups of 16 lanes.  A K or V row of one
+// head is 128 fp16 = 256 bytes = 16 lanes x 128-bit, so a group owns a row and a lane owns 8 channels.
+// Each group asks for its 2 or 4 K rows and V rows before any of them is used, the dot products are
+// reduced over the 16 lanes, and an fp32 online softmax (base 2) keeps (m, l, o[8]) per lane.  Groups
+// are merged through LDS; when a head is cut into several splits the partial (m, l, o[128]) go to
+// the workspace and the last workgroup to arrive for that head merges them, so there is no second
+// launch (from 24 splits on the merge is a short launch of its own).
 #include "attend.h"
 #include "split_merge.h"
 #include "workspace.h"
@@ -14,16 +14,16 @@
 namespace adamas {
 
 constexpr int kTile = 8;             // rows per group per tile, at most
-// A workgroup has 256 or 512 threads = 16 or 32 groups of 16 lanes; a group has 2, 4 or 8 rows in
-// flight, and a split is one such round of loads.  One CU gathers scattered rows slowly (a single
-// 1024-thread workgroup per head takes 25 us for 1024 rows, eight splits 13 us), a group finishes
-// sooner the fewer rows it has to ask for, and publishing a partial result costs about a
-// microsecond.  Hence: 32 groups from 65 rows on; up to 128 rows one split (4 rows per group, no
-// merge); up to 512 rows splits of 64 rows (2 per group, at most 8 splits); up to 2048 rows splits
-// of 128 (at most 16); beyond that splits of 256.  Measured at 32 heads, rows = 128 / 256 / 512 /
-// 1024 / 2048 / 4096, in us: 5.8 / 6.5 / 7.4 / 9.7 / 14.2 / 20.6 (with 16 groups of 8 rows and splits
-// of 128 rows up to 1024 rows, 256 beyond: 7.5 / 9.5 / 10.1 / 12.4 / 15.8 / 20.6).
-constexpr uint32_t kWideRowsFrom = 65;
+// A workgroup has 256, 512 or 1024 threads = 16, 32 or 64 groups of 16 lanes; a group has 2 or 4
+// rows in flight, and a split is one such round of loads.  One CU gathers scattered rows slowly (a
+// single workgroup per head takes 25 us for 1024 rows), a group finishes sooner the fewer rows it
+// has to ask for, and publishing a partial result costs about a microsecond.  Hence: up to 64 rows
+// 16 groups of 4, up to 128 rows 32 groups of 4 (one split, no merge, no workspace); up to 512 rows
+// splits of 64 rows (32 groups of 2, at most 8 splits); up to 2048 rows splits of 128 (64 groups of
+// 2, at most 16); beyond that splits of 256 (64 groups of 4).  Measured at 32 heads, rows = 128 /
+// 256 / 512 / 1024 / 2048 / 4096, in us: 5.8 / 6.5 / 7.4 / 9.3 / 13.5 / 18.8 (with 16 groups of 8
+// rows and splits of 128 rows up to 1024 rows, 32 groups of 8 beyond: 7.5 / 9.5 / 10.1 / 12.4 / 15.8
+// / 20.6).
 constexpr uint32_t kDeferredMergeSplits = 24;  // splits from which the partials get a merge launch
 // (measured at 32768 tokens, 32 heads: 16 splits 14.7 us merged inside the launch, 15.8 us with a merge
 // launch; 32 splits 26.6 against 22.5 us)
@@ -881,11 +881,11 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
     return merge_launch();
   }
   const uint32_t n_rows = sel_idx ? n_sel + 1u : max_seq_len;
-  // one round of loads per split (see the rule at kWideRowsFrom; up to 128 rows that is a single
+  // one round of loads per split (see the rule at kTile; up to 128 rows that is a single
   // split, which needs no workspace), more where that would take more than kMaxSplits splits
-  const bool wide = n_rows >= kWideRowsFrom;
-  const uint32_t tile = n_rows <= 128 ? 4u : n_rows <= 512 ? 2u : n_rows <= 2048 ? 4u : 8u;
-  const uint32_t rows_per_iter = (wide ? 32u : 16u) * tile;
+  const uint32_t threads = n_rows <= 64 ? 256u : n_rows <= 512 ? 512u : 1024u;
+  const uint32_t tile = n_rows <= 128 ? 4u : n_rows <= 2048 ? 2u : 4u;
+  const uint32_t rows_per_iter = threads / 16u * tile;
   uint32_t rows_per_split = rows_per_iter;
   uint32_t n_split = (n_rows + rows_per_split - 1) / rows_per_split;
   if (n_split > kMaxSplits) {
@@ -912,14 +912,16 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
                      static_cast<__half*>(out), partial, counters, num_heads, num_kv_heads,      \
                      page_size, scale_log2, rows_per_split, deferred)
 #define ADAMAS_LAUNCH_SPARSE_L(BF, HND)          \
-  if (!wide) {                                   \
+  if (threads == 256) {                          \
     ADAMAS_LAUNCH_SPARSE_T(BF, HND, 256, 4);     \
-  } else if (tile == 2) {                        \
-    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512, 2);     \
-  } else if (tile == 4) {                        \
+  } else if (threads == 512 && tile == 4) {      \
     ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512, 4);     \
+  } else if (threads == 512) {                   \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512, 2);     \
+  } else if (tile == 2) {                        \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 1024, 2);    \
   } else {                                       \
-    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 512, 8);     \
+    ADAMAS_LAUNCH_SPARSE_T(BF, HND, 1024, 4);    \
   }
 #define ADAMAS_LAUNCH_SPARSE(BF)        \
   if (flags & ADAMAS_F_HND) {           \
