@@ -295,6 +295,28 @@ def test_sparse_attention_page_size_sweep(gpu_device, kv_len, budget, page_size)
         assert np.abs(T.np16(o_f).astype(np.float64) - T.np16(o3).astype(np.float64)).max() <= ATTN_TOL
 
 
+# the operator picks workgroup size, rows per lane group and rows per split from the row count: both
+# sides of every boundary of that rule, random indices, twice in a row (arrival counters back at zero)
+@pytest.mark.parametrize("budget", [64, 65, 128, 129, 512, 513, 1024, 2048, 2049, 3000])
+def test_sparse_attention_row_count_boundaries(gpu_device, budget):
+    kv_len = 4100
+    g = torch.Generator().manual_seed(budget)
+    q = torch.randn(32, 128, generator=g).half()
+    k = torch.randn(kv_len, 32, 128, generator=g).half()
+    v = torch.randn(kv_len, 32, 128, generator=g).half()
+    ctrl = T.make_controller(gpu_device, kv_len, budget, 16, shuffle_seed=budget)
+    kd, vd, qd = k.to(gpu_device), v.to(gpu_device), q.to(gpu_device)
+    T.fill_sequence(ctrl, kd[:kv_len - 1], vd[:kv_len - 1])
+    T.decode_append(ctrl, qd[None], kd[kv_len - 1:], vd[kv_len - 1:])
+    sel = torch.stack([torch.randperm(kv_len - 1, generator=g)[:budget - 1] for _ in range(32)]).int()
+    o = U.decode_sparse_attn(qd[None], ctrl, 0, sel.to(gpu_device))
+    sets = [np.append(sel[h].numpy(), kv_len - 1) for h in range(32)]
+    want = O.sparse_attention(T.np16(q), T.np16(k), T.np16(v), sets)
+    assert np.abs(T.np16(o)[0].astype(np.float64) - want).max() <= ATTN_TOL
+    o2 = U.decode_sparse_attn(qd[None], ctrl, 0, sel.to(gpu_device))
+    assert torch.equal(o, o2)
+
+
 @pytest.mark.parametrize("kv_len", [1, 2, 129, 4000, 9000])
 def test_dense_mode_equals_dense_attention(gpu_device, kv_len):
     seq = synth.make_sequence(kv_len, 0, torch.Generator().manual_seed(kv_len))
