@@ -783,7 +783,14 @@ static int sparse_decode_impl(const void* q, const void* kv_data, const int32_t*
   // 8 query heads = 8 / gq key/value heads); other group sizes run the per-query-head kernels, whose
   // lanes of one group load the same rows (correct, merged by the memory pipeline, but slower)
   const bool gqa_kernel = (gq == 2 || gq == 4 || gq == 8) && num_heads % kDenseHeads == 0;
-  if (!sel_idx && num_heads % kDenseHeads == 0) {
+  // Short sequences attend all their tokens through the kernel for row lists below (sel_idx ==
+  // nullptr: the rows are the positions 0 .. seq_len - 1): the dense kernels cut a sequence into
+  // splits of at least 128 tokens for eight heads at once, which leaves most CUs idle when the
+  // sequence is short (1024 tokens: 17.5 us against 9.4; 130 tokens: 16.4 against 7.1; equal at
+  // 4096 tokens; with four query heads per key/value head, whose rows the row kernel reads four
+  // times, 14.3 against 8.6 us at 1024 tokens and 11.8 at 2048).
+  const uint32_t dense_rows_limit = gq == 1 ? 4096u : 2048u;
+  if (!sel_idx && num_heads % kDenseHeads == 0 && max_seq_len > dense_rows_limit) {
     // dense: kDenseTargetBlocks workgroups, at least 128 tokens per split
     const uint32_t groups = batch * (num_heads / kDenseHeads);
     // grouped queries read 1/gq of the bytes per unit of arithmetic: there the kernel is bound by

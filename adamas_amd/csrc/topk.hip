@@ -14,15 +14,20 @@
 //              makes the candidates visible, no atomics or fences are involved.
 //   k > 1024   one workgroup of 1024 threads per row streams the row once per bisection round.
 //
-// Integer keys (the distances of the estimator, ADAMAS_KEY_*_INT) with k <= 255 and rows longer than
-// 4096 take the two-level scheme of chunk_select.h instead, the one the fused decode step uses: a
-// launch of one WAVE per chunk of 512-2048 keys (threshold of the chunk from a histogram in LDS, 2048
-// waves for 32 rows of 32768), then one workgroup per row that gets the threshold from the summed chunk
-// histograms.  Two short launches instead of one long one with 32 workgroups.  Integer keys with a
-// larger k (or rows too long for the candidate lists) take the histogram scheme at the end of this
-// file: the same two launches, with plain 512-bin counts per chunk instead of candidate lists.
+// Integer keys (the distances of the estimator, ADAMAS_KEY_*_INT) with k <= 255 take the two-level
+// scheme the fused decode step uses, given a workspace: a launch of one WAVE per chunk of 512-2048
+// keys (threshold of the chunk from a histogram in LDS, 2048 waves for 32 rows of 32768) that writes
+// a short list of the chunk's smallest keys, then one workgroup per row that reads the threshold off
+// a histogram of the listed keys and goes back to the input for the rare chunk whose list ran out.
+// Two short launches: 6.1 us for 32 rows of 32768 keys at k = 127, against 9.6 us with lists of the
+// full k and 21 us for the bisection kernels; also faster than the single launch for short rows
+// (4096 keys: 5.9 against 9.5 us).  Rows beyond 131072 keys keep lists of the full k and a histogram
+// row per chunk (select_chunks_int_kernel, select_final_int_kernel).  Integer keys with a larger k
+// take the histogram scheme at the end of this file: the same two launches, with plain 512-bin
+// counts per chunk instead of candidate lists.
 #include "chunk_select.h"
 #include "select.h"
+#include "workspace.h"
 
 namespace adamas {
 
@@ -385,6 +390,280 @@ __global__ __launch_bounds__(kFinalThreads) void select_final_int_kernel(
   }
 }
 
+// ---- integer keys, k <= 255, rows of up to 131072 keys: short candidate lists ------------------------
+// The scheme of the fused decode step (fused_step.hip).  Level 1: one wave per chunk of 512 - 2048
+// keys (at most 64 chunks per row) writes the kc = 16 .. 256 smallest keys of its chunk, ties to the
+// lowest index: a chunk holds k / chunks of the selection on average, so lists of the full k would be
+// mostly padding (64 x 128 slots for 127 winners).  Level 2: one workgroup per row builds a histogram
+// of the listed keys in LDS, reads threshold and tie quota off it and ranks the listed candidates
+// with prefix scans.  A list is a prefix of its chunk in (key, index) order: if its last entry is not
+// selected, nothing the chunk left out can be.  If it is, and the chunk holds more keys than the
+// list, the workgroup takes that chunk's keys from the input row again and selects among all of them,
+// so the result is exact for any input (at most k / kc chunks can need that).
+constexpr uint32_t kCapMaxChunks = 64;       // the flags of all chunks fit one ballot
+constexpr uint32_t kCapMaxRowLen = kCapMaxChunks * 2048;
+constexpr uint32_t kCapSlots = 2 * kFinalThreads;  // candidate slots per row: two per thread of level 2
+
+struct CapLayout {
+  uint32_t ok;
+  uint32_t items;      // keys per lane at level 1: 8, 16 or 32
+  uint32_t n_chunks;   // <= kCapMaxChunks
+  uint32_t kc, kc_log2;
+  size_t cand_bytes;
+};
+
+static CapLayout cap_layout(uint32_t num_rows, uint32_t n_max, uint32_t k) {
+  CapLayout L{};
+  if (k == 0 || k > kIntMaxK || n_max == 0 || n_max > kCapMaxRowLen) return L;
+  L.items = 8;
+  while (ceil_div(n_max, kWave * L.items) > kCapMaxChunks) L.items *= 2;
+  L.n_chunks = ceil_div(n_max, kWave * L.items);
+  L.kc = std::max(8u, std::min(pow2_floor(kCapSlots / L.n_chunks), pow2_ceil(k)));
+  while ((1u << L.kc_log2) < L.kc) ++L.kc_log2;
+  L.cand_bytes = (static_cast<size_t>(num_rows) * L.n_chunks * L.kc * 8 + 255) / 256 * 256;
+  L.ok = 1;
+  return L;
+}
+
+// level 1: grid (ceil(n_chunks / 8), rows), 512 threads; wave w takes chunk blockIdx.x * 8 + w
+template <int kItems, int kKeyMode>
+__global__ __launch_bounds__(kIntWaves* kWave) void select_chunks_capped_kernel(
+    SelectArgs a, uint64_t* __restrict__ cand, uint32_t n_chunks, uint32_t kc) {
+  const uint32_t key_mode = kKeyMode >= 0 ? static_cast<uint32_t>(kKeyMode) : a.key_mode;
+  const bool vec_ok = kKeyMode >= 0 || a.vec_ok != 0;
+  __shared__ alignas(16) uint32_t hist_lds[kIntWaves][kChunkHistWords];
+  __shared__ alignas(16) uint32_t key_lds[kIntWaves][kWave * kItems / 2];  // two keys per word
+  const int lane = lane_id();
+  const int wave = wave_id_uniform();
+  const uint32_t row = blockIdx.y;
+  const uint32_t chunk = blockIdx.x * kIntWaves + static_cast<uint32_t>(wave);
+  if (chunk >= n_chunks) return;  // whole waves leave; nothing below synchronises the workgroup
+  constexpr uint32_t kChunk = kWave * kItems;
+  const uint32_t chunk_base = chunk * kChunk;
+  const uint32_t n = row_length(a, row);
+  uint64_t* dst = cand + (static_cast<size_t>(row) * n_chunks + chunk) * kc;
+  if (chunk_base >= n) {
+    for (uint32_t i = lane; i < kc; i += kWave) dst[i] = kEmptyCand64;
+    return;
+  }
+  const uint16_t* vrow = a.values + static_cast<int64_t>(row) * a.row_stride;
+  uint32_t keys[kItems];
+#pragma unroll
+  for (int j = 0; j < kItems / 8; ++j)
+    load_value_keys(vrow, chunk_base + static_cast<uint32_t>(lane) * kItems + j * 8, n,
+                    vec_ok, key_mode, &keys[j * 8]);
+  // a listed key is picked by a run-time index: the keys of the chunk go to LDS, item order
+  // (the LDS operations of one wave are carried out in order, so the wave reads them back below
+  // without a barrier)
+  uint32_t* kl = key_lds[wave] + lane * (kItems / 2);
+#pragma unroll
+  for (int j = 0; j < kItems / 8; ++j)
+    *reinterpret_cast<uint4*>(kl + 4 * j) =
+        make_uint4((keys[8 * j] & 0xffffu) | (keys[8 * j + 1] << 16),
+                   (keys[8 * j + 2] & 0xffffu) | (keys[8 * j + 3] << 16),
+                   (keys[8 * j + 4] & 0xffffu) | (keys[8 * j + 5] << 16),
+                   (keys[8 * j + 6] & 0xffffu) | (keys[8 * j + 7] << 16));
+  const int32_t* irow =
+      a.in_idx ? a.in_idx + static_cast<int64_t>(row) * a.in_idx_stride : nullptr;
+  const uint16_t* kl16 = reinterpret_cast<const uint16_t*>(key_lds[wave]);
+  chunk_select_capped<kItems, true>(
+      keys, kc, dst, hist_lds[wave],
+      [&](uint32_t item) __attribute__((always_inline)) -> uint32_t { return kl16[item]; },
+      [&](uint32_t item) __attribute__((always_inline)) -> uint32_t {
+        const uint32_t e = chunk_base + item;
+        return irow ? static_cast<uint32_t>(irow[e]) : e;
+      });
+}
+
+struct CapFinalShared {
+  alignas(16) uint32_t hist[kHistBins];      // listed candidates per key value
+  alignas(16) uint32_t wclass[kFinalWaves];  // per-wave class totals of the rank scan: below | tied << 16
+  uint32_t flag[kCapMaxChunks];              // chunks whose list ran out (taken from the row again)
+  uint32_t any_flag;
+  uint32_t fb[kCapMaxChunks], ft[kCapMaxChunks];  // their keys below / equal to the threshold
+  uint32_t tbase[kCapMaxChunks];             // tied list entries of all chunks before them
+  int32_t idx[kIntMaxK + 1];
+  uint16_t val[kIntMaxK + 1];
+};
+
+// level 2: grid (rows), 512 threads, two candidate slots per thread
+__global__ __launch_bounds__(kFinalThreads) void select_final_capped_kernel(
+    SelectArgs a, const uint64_t* __restrict__ cand, uint32_t n_chunks, uint32_t kc_log2,
+    uint32_t chunk_keys) {
+  static_assert(kFinalThreads == kHistBins, "one thread per key value");
+  static_assert(kFinalWaves == 8, "two 128-bit reads cover the wave totals");
+  static_assert(kCapMaxChunks == kWave, "the flags of all chunks fit one ballot");
+  __shared__ CapFinalShared sh;
+  const uint32_t row = blockIdx.x;
+  const uint32_t tid = threadIdx.x;
+  const int lane = lane_id();
+  const int wave = wave_id_uniform();
+  const uint32_t kc = 1u << kc_log2;
+  const uint32_t n_slots = n_chunks << kc_log2;
+  const uint64_t* crow = cand + static_cast<size_t>(row) * n_slots;
+  const uint32_t slot0 = 2u * tid;
+  const bool have = slot0 < n_slots;
+  uint4 raw = make_uint4(~0u, ~0u, ~0u, ~0u);  // an unused slot is all ones
+  if (have) raw = *reinterpret_cast<const uint4*>(crow + slot0);
+  const uint32_t n = row_length(a, row);
+  const uint32_t k = a.k;
+  sh.hist[tid] = 0u;
+  if (tid < kCapMaxChunks) sh.flag[tid] = 0u;
+  if (tid == 0) sh.any_flag = 0u;
+  // a candidate is (key << 48) | (item index in its chunk << 32) | payload
+  uint32_t key[2] = {raw.y >> 16, raw.w >> 16};  // an unused slot reads 0xffff: above every threshold
+  const uint32_t pay[2] = {raw.x, raw.z};
+  const uint32_t chunk_mine = slot0 >> kc_log2;
+  __syncthreads();  // the histogram is cleared
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (key[i] < static_cast<uint32_t>(kHistBins)) atomicAdd(&sh.hist[key[i]], 1u);
+  __syncthreads();  // the histogram is complete
+  WavePlan plan = wave_plan_from_hist(sh.hist, k);  // every wave for itself
+  uint32_t rb, re, list_below;
+  auto rank_slots = [&]() __attribute__((always_inline)) {
+    uint32_t mine = 0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      mine += (key[i] < plan.thr ? 1u : 0u) + ((key[i] == plan.thr ? 1u : 0u) << 16);
+    const uint32_t incl = wave_inclusive_scan_dpp(mine);
+    if (lane == kWave - 1) sh.wclass[wave] = incl;
+    __syncthreads();
+    const uint4 lo = *reinterpret_cast<const uint4*>(&sh.wclass[0]);
+    const uint4 hi = *reinterpret_cast<const uint4*>(&sh.wclass[4]);
+    const uint32_t t[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    uint32_t before = 0, all = 0;  // the 16-bit fields cannot carry: at most 1024 slots
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      before += w < wave ? t[w] : 0u;
+      all += t[w];
+    }
+    const uint32_t excl = before + incl - mine;
+    rb = excl & 0xffffu;
+    re = excl >> 16;
+    list_below = all & 0xffffu;
+  };
+  const bool as_half = a.key_mode == ADAMAS_KEY_FP16_INT;
+  auto put = [&](uint32_t pos, uint32_t kv, uint32_t payload) __attribute__((always_inline)) {
+    sh.idx[pos] = static_cast<int32_t>(payload);
+    // the key in the format of the input: integer keys are their own value
+    sh.val[pos] = as_half ? __half_as_ushort(__float2half_rn(static_cast<float>(kv)))
+                          : static_cast<uint16_t>(kv);
+  };
+  auto emit_slots = [&](uint32_t tie_shift) __attribute__((always_inline)) -> bool {
+    uint32_t pb = rb, pe = re + tie_shift;
+    bool last_selected = false;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const bool is_b = key[i] < plan.thr, is_e = key[i] == plan.thr;
+      const bool take = is_b || (is_e && pe < plan.quota);
+      if (take) put(is_b ? pb : plan.n_below + pe, key[i], pay[i]);
+      pb += is_b ? 1u : 0u;
+      pe += is_e ? 1u : 0u;
+      last_selected = take;
+    }
+    return last_selected;
+  };
+  auto chunk_len = [&](uint32_t c) __attribute__((always_inline)) -> uint32_t {
+    const uint32_t t0 = c * chunk_keys;
+    return t0 < n ? min(chunk_keys, n - t0) : 0u;
+  };
+  rank_slots();
+  {
+    const bool last_selected = emit_slots(0u);
+    if (last_selected && ((slot0 + 1u) & (kc - 1u)) == kc - 1u && chunk_len(chunk_mine) > kc) {
+      sh.flag[chunk_mine] = 1u;
+      sh.any_flag = 1u;
+    }
+  }
+  __syncthreads();  // the output list is complete, or some chunk is flagged
+
+  if (sh.any_flag) {
+    const uint16_t* vrow = a.values + static_cast<int64_t>(row) * a.row_stride;
+    const int32_t* irow =
+        a.in_idx ? a.in_idx + static_cast<int64_t>(row) * a.in_idx_stride : nullptr;
+    const uint32_t key_mode = a.key_mode;
+    const uint64_t fmask = __ballot(sh.flag[lane] != 0u);  // the same in every wave
+    const bool mine_flagged = have && ((fmask >> chunk_mine) & 1ull) != 0;
+    if (mine_flagged) {  // the listed entries of such a chunk leave the count: its keys come back below
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (key[i] < static_cast<uint32_t>(kHistBins)) atomicSub(&sh.hist[key[i]], 1u);
+        key[i] = 0xffffu;
+      }
+    }
+    for (uint64_t m = fmask; m; m &= m - 1) {
+      const uint32_t c = static_cast<uint32_t>(__ffsll(static_cast<long long>(m)) - 1);
+      const uint32_t t0 = c * chunk_keys, len = chunk_len(c);
+      for (uint32_t t = tid; t < len; t += kFinalThreads)
+        atomicAdd(&sh.hist[make_key(vrow[t0 + t], key_mode)], 1u);
+    }
+    __syncthreads();  // counts complete
+    plan = wave_plan_from_hist(sh.hist, k);
+    // wave w counts the keys below / equal to the new threshold in the flagged chunks w, w+8, ...
+    {
+      uint32_t f = 0;
+      for (uint64_t m = fmask; m; m &= m - 1, ++f) {
+        if ((f & (kFinalWaves - 1)) != static_cast<uint32_t>(wave)) continue;
+        const uint32_t c = static_cast<uint32_t>(__ffsll(static_cast<long long>(m)) - 1);
+        const uint32_t t0 = c * chunk_keys, len = chunk_len(c);
+        uint32_t cb = 0, ce = 0;
+        for (uint32_t t = 0; t < len; t += kWave) {
+          const uint32_t d = t + lane < len ? make_key(vrow[t0 + t + lane], key_mode) : 0xffffu;
+          cb += __popcll(__ballot(d < plan.thr));
+          ce += __popcll(__ballot(d == plan.thr));
+        }
+        if (lane == 0) {
+          sh.fb[c] = cb;
+          sh.ft[c] = ce;
+        }
+      }
+    }
+    rank_slots();  // (its barrier also publishes fb and ft)
+    // listed ties of all chunks in front of a flagged chunk: what its first slot's thread counted
+    if (mine_flagged && (slot0 & (kc - 1u)) == 0u) sh.tbase[chunk_mine] = re;
+    uint32_t tie_shift = 0;  // tied keys of flagged chunks in front of this thread's chunk
+    for (uint64_t m = have ? fmask & ((1ull << chunk_mine) - 1ull) : 0ull; m; m &= m - 1)
+      tie_shift += sh.ft[__ffsll(static_cast<long long>(m)) - 1];
+    __syncthreads();
+    emit_slots(tie_shift);
+    // the flagged chunks, walked in index order by their waves: keys below the threshold go behind
+    // the listed ones, tied keys take the rank their index gives them among all ties
+    {
+      uint32_t f = 0, bb = list_below, tb = 0;
+      for (uint64_t m = fmask; m; m &= m - 1, ++f) {
+        const uint32_t c = static_cast<uint32_t>(__ffsll(static_cast<long long>(m)) - 1);
+        if ((f & (kFinalWaves - 1)) == static_cast<uint32_t>(wave)) {
+          const uint32_t t0 = c * chunk_keys, len = chunk_len(c);
+          uint32_t pb = bb, pe = sh.tbase[c] + tb;
+          for (uint32_t t = 0; t < len; t += kWave) {
+            const uint32_t e = t0 + t + lane;
+            const uint32_t d = t + lane < len ? make_key(vrow[e], key_mode) : 0xffffu;
+            const uint64_t mb = __ballot(d < plan.thr), me = __ballot(d == plan.thr);
+            const uint32_t r_e = pe + lanes_below(me);
+            const bool is_b = d < plan.thr;
+            if (is_b || (d == plan.thr && r_e < plan.quota))
+              put(is_b ? pb + lanes_below(mb) : plan.n_below + r_e, d,
+                  irow ? static_cast<uint32_t>(irow[e]) : e);
+            pb += __popcll(mb);
+            pe += __popcll(me);
+          }
+        }
+        bb += sh.fb[c];
+        tb += sh.ft[c];
+      }
+    }
+    __syncthreads();  // the output list is complete
+  }
+  const uint32_t n_take = plan.n_take;
+  int32_t* oi = a.out_idx + static_cast<int64_t>(row) * a.out_stride;
+  uint16_t* ov = a.out_vals ? a.out_vals + static_cast<int64_t>(row) * a.out_stride : nullptr;
+  for (uint32_t i = tid; i < k; i += kFinalThreads) {
+    oi[i] = i < n_take ? sh.idx[i] : -1;
+    if (ov) ov[i] = i < n_take ? sh.val[i] : static_cast<uint16_t>(0);
+  }
+}
+
 // ---- integer keys, any k: chunk histograms, then threshold and emission ------------------------------
 // Integer keys take 512 values, so the k-th smallest key of a row can be read off a histogram instead
 // of being searched for.  Level 1 (one wave per chunk of 1024 keys, the row spread over many CUs)
@@ -742,8 +1021,10 @@ using namespace adamas;
 extern "C" size_t adamas_topk_workspace_bytes(uint32_t num_rows, uint32_t n_max, uint32_t k) {
   const IntLayout il = int_layout(num_rows, n_max, k);
   size_t int_bytes = il.ok ? il.cand_bytes + il.hist_bytes : 0;  // two-level integer path
+  const CapLayout cl = cap_layout(num_rows, n_max, k);
   // integer keys outside its reach (k above 255, very long rows): chunk histograms
   if (!il.ok && n_max > kChunkItems) int_bytes = hist_path_bytes(num_rows, n_max);
+  if (cl.ok && cl.cand_bytes > int_bytes) int_bytes = cl.cand_bytes;
   if (k > kChunkedMaxK || n_max <= kFinalItems) return int_bytes > 256 ? int_bytes : 256;
   size_t slots = 0;
   uint32_t n = n_max;
@@ -787,8 +1068,41 @@ extern "C" int adamas_topk(const void* values, int64_t row_stride, uint32_t n_ma
   a.out_vals = static_cast<uint16_t*>(out_vals);
   a.out_stride = out_stride;
 
-  // integer keys: two short launches (one wave per chunk, then one workgroup per row), when the
-  // caller's workspace holds the candidate lists; otherwise the general paths below
+  // integer keys, k <= 255, rows up to 131072 keys: short candidate lists per chunk, then one
+  // workgroup per row (two short launches), when the caller's workspace holds the lists
+  const CapLayout cl = cap_layout(num_rows, n_max, k);
+  if (cl.ok && key_mode != ADAMAS_KEY_FP16_GENERIC && workspace &&
+      workspace_bytes >= cl.cand_bytes && (reinterpret_cast<uintptr_t>(workspace) & 255) == 0) {
+    uint64_t* cand = static_cast<uint64_t*>(workspace);
+    const dim3 grid1(ceil_div(cl.n_chunks, kIntWaves), num_rows);
+#define ADAMAS_LAUNCH_CHUNKS_CAP(ITEMS, MODE)                                                       \
+  hipLaunchKernelGGL((select_chunks_capped_kernel<ITEMS, MODE>), grid1, dim3(kIntWaves * kWave), 0, \
+                     s, a, cand, cl.n_chunks, cl.kc)
+#define ADAMAS_LAUNCH_CHUNKS_CAP_MODE(ITEMS)                                \
+  if (a.vec_ok && key_mode == ADAMAS_KEY_FP16_INT) {                        \
+    ADAMAS_LAUNCH_CHUNKS_CAP(ITEMS, static_cast<int>(ADAMAS_KEY_FP16_INT)); \
+  } else if (a.vec_ok && key_mode == ADAMAS_KEY_U16_INT) {                  \
+    ADAMAS_LAUNCH_CHUNKS_CAP(ITEMS, static_cast<int>(ADAMAS_KEY_U16_INT));  \
+  } else {                                                                  \
+    ADAMAS_LAUNCH_CHUNKS_CAP(ITEMS, -1);                                    \
+  }
+    if (cl.items == 8) {
+      ADAMAS_LAUNCH_CHUNKS_CAP_MODE(8)
+    } else if (cl.items == 16) {
+      ADAMAS_LAUNCH_CHUNKS_CAP_MODE(16)
+    } else {
+      ADAMAS_LAUNCH_CHUNKS_CAP_MODE(32)
+    }
+#undef ADAMAS_LAUNCH_CHUNKS_CAP_MODE
+#undef ADAMAS_LAUNCH_CHUNKS_CAP
+    ADAMAS_RETURN_IF_LAUNCH_FAILED();
+    hipLaunchKernelGGL(select_final_capped_kernel, dim3(num_rows), dim3(kFinalThreads), 0, s, a, cand,
+                       cl.n_chunks, cl.kc_log2, kWave * cl.items);
+    ADAMAS_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  // the same with lists of the full k and a histogram row per chunk (rows beyond 131072 keys): when
+  // the caller's workspace holds them; otherwise the general paths below
   const IntLayout il = int_layout(num_rows, n_max, k);
   if (il.ok && key_mode != ADAMAS_KEY_FP16_GENERIC && workspace &&
       workspace_bytes >= il.cand_bytes + il.hist_bytes &&
