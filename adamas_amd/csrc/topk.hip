@@ -482,6 +482,7 @@ struct CapFinalShared {
   uint32_t any_flag;
   uint32_t fb[kCapMaxChunks], ft[kCapMaxChunks];  // their keys below / equal to the threshold
   uint32_t tbase[kCapMaxChunks];             // tied list entries of all chunks before them
+  uint32_t bbase[kCapMaxChunks];             // list entries below the threshold of all chunks before them
   int32_t idx[kIntMaxK + 1];
   uint16_t val[kIntMaxK + 1];
 };
@@ -520,7 +521,7 @@ __global__ __launch_bounds__(kFinalThreads) void select_final_capped_kernel(
     if (key[i] < static_cast<uint32_t>(kHistBins)) atomicAdd(&sh.hist[key[i]], 1u);
   __syncthreads();  // the histogram is complete
   WavePlan plan = wave_plan_from_hist(sh.hist, k);  // every wave for itself
-  uint32_t rb, re, list_below;
+  uint32_t rb, re;
   auto rank_slots = [&]() __attribute__((always_inline)) {
     uint32_t mine = 0;
 #pragma unroll
@@ -532,16 +533,12 @@ __global__ __launch_bounds__(kFinalThreads) void select_final_capped_kernel(
     const uint4 lo = *reinterpret_cast<const uint4*>(&sh.wclass[0]);
     const uint4 hi = *reinterpret_cast<const uint4*>(&sh.wclass[4]);
     const uint32_t t[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    uint32_t before = 0, all = 0;  // the 16-bit fields cannot carry: at most 1024 slots
+    uint32_t before = 0;  // the 16-bit fields cannot carry: at most 1024 slots
 #pragma unroll
-    for (int w = 0; w < 8; ++w) {
-      before += w < wave ? t[w] : 0u;
-      all += t[w];
-    }
+    for (int w = 0; w < 8; ++w) before += w < wave ? t[w] : 0u;
     const uint32_t excl = before + incl - mine;
     rb = excl & 0xffffu;
     re = excl >> 16;
-    list_below = all & 0xffffu;
   };
   const bool as_half = a.key_mode == ADAMAS_KEY_FP16_INT;
   auto put = [&](uint32_t pos, uint32_t kv, uint32_t payload) __attribute__((always_inline)) {
@@ -550,8 +547,8 @@ __global__ __launch_bounds__(kFinalThreads) void select_final_capped_kernel(
     sh.val[pos] = as_half ? __half_as_ushort(__float2half_rn(static_cast<float>(kv)))
                           : static_cast<uint16_t>(kv);
   };
-  auto emit_slots = [&](uint32_t tie_shift) __attribute__((always_inline)) -> bool {
-    uint32_t pb = rb, pe = re + tie_shift;
+  auto emit_slots = [&](uint32_t below_shift, uint32_t tie_shift) __attribute__((always_inline)) -> bool {
+    uint32_t pb = rb + below_shift, pe = re + tie_shift;
     bool last_selected = false;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -570,7 +567,7 @@ __global__ __launch_bounds__(kFinalThreads) void select_final_capped_kernel(
   };
   rank_slots();
   {
-    const bool last_selected = emit_slots(0u);
+    const bool last_selected = emit_slots(0u, 0u);
     if (last_selected && ((slot0 + 1u) & (kc - 1u)) == kc - 1u && chunk_len(chunk_mine) > kc) {
       sh.flag[chunk_mine] = 1u;
       sh.any_flag = 1u;
@@ -620,22 +617,29 @@ __global__ __launch_bounds__(kFinalThreads) void select_final_capped_kernel(
       }
     }
     rank_slots();  // (its barrier also publishes fb and ft)
-    // listed ties of all chunks in front of a flagged chunk: what its first slot's thread counted
-    if (mine_flagged && (slot0 & (kc - 1u)) == 0u) sh.tbase[chunk_mine] = re;
-    uint32_t tie_shift = 0;  // tied keys of flagged chunks in front of this thread's chunk
-    for (uint64_t m = have ? fmask & ((1ull << chunk_mine) - 1ull) : 0ull; m; m &= m - 1)
-      tie_shift += sh.ft[__ffsll(static_cast<long long>(m)) - 1];
+    // listed entries of all chunks in front of a flagged chunk: what its first slot's thread counted
+    if (mine_flagged && (slot0 & (kc - 1u)) == 0u) {
+      sh.tbase[chunk_mine] = re;
+      sh.bbase[chunk_mine] = rb;
+    }
+    // keys of flagged chunks in front of this thread's chunk, by class
+    uint32_t tie_shift = 0, below_shift = 0;
+    for (uint64_t m = have ? fmask & ((1ull << chunk_mine) - 1ull) : 0ull; m; m &= m - 1) {
+      const int fc = __ffsll(static_cast<long long>(m)) - 1;
+      tie_shift += sh.ft[fc];
+      below_shift += sh.fb[fc];
+    }
     __syncthreads();
-    emit_slots(tie_shift);
-    // the flagged chunks, walked in index order by their waves: keys below the threshold go behind
-    // the listed ones, tied keys take the rank their index gives them among all ties
+    emit_slots(below_shift, tie_shift);
+    // the flagged chunks, walked in index order by their waves: every key takes the rank its index
+    // gives it within its class, among listed entries and keys of flagged chunks alike
     {
-      uint32_t f = 0, bb = list_below, tb = 0;
+      uint32_t f = 0, bb = 0, tb = 0;
       for (uint64_t m = fmask; m; m &= m - 1, ++f) {
         const uint32_t c = static_cast<uint32_t>(__ffsll(static_cast<long long>(m)) - 1);
         if ((f & (kFinalWaves - 1)) == static_cast<uint32_t>(wave)) {
           const uint32_t t0 = c * chunk_keys, len = chunk_len(c);
-          uint32_t pb = bb, pe = sh.tbase[c] + tb;
+          uint32_t pb = sh.bbase[c] + bb, pe = sh.tbase[c] + tb;
           for (uint32_t t = 0; t < len; t += kWave) {
             const uint32_t e = t0 + t + lane;
             const uint32_t d = t + lane < len ? make_key(vrow[e], key_mode) : 0xffffu;

@@ -231,6 +231,72 @@ def test_topk_two_level_integer_path(gpu_device, n, k, mode):
         assert torch.equal(idx, out2)
 
 
+@pytest.mark.parametrize("mode", ["fp16", "u16"])
+@pytest.mark.parametrize("kind", ["equal", "clustered", "runs", "short_rows"])
+@pytest.mark.parametrize("n,k", [(32768, 127), (33000, 127), (131072, 255), (5000, 63), (70000, 255),
+                                 (20000, 16), (600, 200)])
+def test_topk_short_lists_fall_back_to_the_row(gpu_device, n, k, kind, mode):
+    """The chunk lists of the two-level integer selection hold fewer entries than k.  Rows whose
+    selection needs more keys of one chunk than its list holds (every key tied, the smallest keys
+    clustered in one chunk, long runs of equal keys across chunk boundaries, rows that end inside
+    the first chunk) are completed from the input row: positions, order, gathered indices and
+    returned values must equal the general path's."""
+    rng = np.random.default_rng(n * 7 + k)
+    rows = 32
+    if kind == "equal":
+        ints = np.full((rows, n), 37, dtype=np.int64)
+    elif kind == "clustered":
+        ints = rng.integers(200, 385, size=(rows, n))
+        for r in range(rows):
+            start = int(rng.integers(0, max(1, n - 2 * k)))
+            ints[r, start:start + 2 * k] = rng.integers(0, 50, size=min(2 * k, n - start))
+    elif kind == "runs":
+        run = np.repeat(rng.integers(90, 110, size=(rows, n // 300 + 1)), 300, axis=1)[:, :n]
+        ints = run
+    else:
+        ints = rng.integers(0, 385, size=(rows, n))
+    if mode == "fp16":
+        v = torch.from_numpy(ints.astype(np.float16)).to(gpu_device)
+        key_mode = _lib.KEY_FP16_INT
+    else:
+        v = torch.from_numpy(ints.astype(np.uint16).view(np.int16)).to(gpu_device).view(torch.float16)
+        key_mode = _lib.KEY_U16_INT
+    lens = None
+    if kind == "short_rows":   # per-row lengths, some shorter than k, some ending inside chunk 0
+        lens = rng.integers(1, n, size=rows).astype(np.int32)
+        lens[:4] = [1, k - 1, k, k + 1]
+        lens[4] = min(n, 300)
+    perm = torch.stack([torch.randperm(n, generator=torch.Generator().manual_seed(i)) for i in range(rows)])
+    pi = perm.int().to(gpu_device)
+    lib = _lib.load()
+    idx = torch.full((rows, k), -7, dtype=torch.int32, device=gpu_device)
+    val = torch.zeros((rows, k), dtype=torch.float16, device=gpu_device)
+    ws = torch.zeros(lib.adamas_topk_workspace_bytes(rows, n, k), dtype=torch.uint8, device=gpu_device)
+    lens_d = torch.from_numpy(lens).to(gpu_device) if lens is not None else None
+    for _ in range(2):   # twice on the same workspace
+        rc = lib.adamas_topk(v.data_ptr(), v.stride(0), n, _lib.ptr(lens_d), 1, 0, pi.data_ptr(), pi.stride(0),
+                             rows, k, idx.data_ptr(), val.data_ptr(), k, key_mode, ws.data_ptr(), ws.numel(),
+                             _lib.current_stream())
+        _lib.check(rc, "adamas_topk")
+    got = idx.cpu().numpy()
+    gval = T.np16(val).astype(np.float32) if mode == "fp16" else T.np16(val).view(np.uint16).astype(np.float32)
+    inv = torch.argsort(perm, dim=1).numpy()
+    for r in range(rows):
+        nr = int(lens[r]) if lens is not None else n
+        row = ints[r, :nr]
+        take = min(k, nr)
+        # ties to the lowest index; output order: keys below the threshold by index, then the ties
+        order = np.lexsort((np.arange(nr), row))[:take]
+        thr = row[order[-1]]
+        want = np.concatenate([np.sort(order[row[order] < thr]), np.sort(order[row[order] == thr])])
+        if nr <= k:   # a row no longer than k is taken whole, in index order
+            want = np.arange(nr)
+        assert (got[r, take:] == -1).all(), (r, nr)
+        pos = inv[r][got[r, :take]]          # undo the gather
+        assert np.array_equal(pos, want), (r, nr)
+        assert np.array_equal(gval[r, :take], row[want].astype(np.float32)), (r, nr)
+
+
 def test_topk_unaligned_rows_and_short_rows(gpu_device):
     rng = np.random.default_rng(3)
     base = torch.from_numpy(rng.integers(0, 385, size=(32 * 1001 + 3,)).astype(np.float16)).to(gpu_device)
