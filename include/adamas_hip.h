@@ -175,10 +175,12 @@ int adamas_estimate(const void* q_code, const void* code_data, const int32_t* pa
  * index order.  out_vals (optional, 2-byte elements, same layout as out_idx) receives the keys.
  * key_mode: one of ADAMAS_KEY_*.  in_idx entries must be non-negative.
  * workspace: adamas_topk_workspace_bytes(num_rows, n_max, k) bytes, 256-byte aligned, zero-filled
- * once after allocation (the library leaves it reusable).  With the integer key modes and rows longer
- * than 4096 it holds, for k <= 255, the candidate lists of a two-level selection (one wave per chunk
- * of 512-2048 keys, then one workgroup per row) and, for larger k, one 512-bin histogram per chunk
- * of 1024 keys (threshold and positions are then read off the histograms).  out_vals holds the key
+ * once after allocation (the library leaves it reusable).  With the integer key modes it holds, for
+ * k <= 255, the candidate lists of a two-level selection (one wave per chunk of 512-2048 keys writes
+ * a short list of the chunk's smallest keys, then one workgroup per row selects among the listed
+ * keys and goes back to the row for a chunk whose list ran out) and, for larger k and rows longer
+ * than 4096, one 512-bin histogram per chunk of 1024 keys (threshold and positions are then read off
+ * the histograms).  out_vals holds the key
  * in the format of the input (integer keys are clamped to 511).  It may be NULL for rows of at most
  * 32768 elements or k > 1024: those are served by one launch with one workgroup per row, which is
  * several times slower for long rows.  The reference passes a scratch buffer too (`buf`).

@@ -83,7 +83,9 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.adamas_topk_workspace_bytes(32, 32767, 127) == 32 * 64 * (128 * 8 + 512)
     # k above 255: one row of 512 16-bit counts per chunk of 1024 keys
     assert lib.adamas_topk_workspace_bytes(32, 32767, 300) == 32 * 32 * 1024
-    assert lib.adamas_topk_workspace_bytes(32, 4096, 127) == 256
+    # short rows, k <= 255: 8 chunks x 128 candidates x 8 B per row (short candidate lists)
+    assert lib.adamas_topk_workspace_bytes(32, 4096, 127) == 32 * 8 * 128 * 8
+    assert lib.adamas_topk_workspace_bytes(32, 4096, 300) == 256       # one launch, no workspace
     assert lib.adamas_sparse_decode(16, 16, 16, 16, 16, None, 0, 0, 16, None, 0, 1, 32, 32, 64, 16, 0.1, 10, None) == -2
     # several splits without a workspace
     assert lib.adamas_sparse_decode(16, 16, 16, 16, 16, None, 0, 0, 16, None, 0, 1, 32, 8, 128, 16, 0.1, 5000, None) == -3
