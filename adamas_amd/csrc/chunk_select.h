@@ -1,15 +1,23 @@
 // Two-level exact selection of the k smallest integer keys (0..511), shared by the fused decode step
 // and the stand-alone top-k (gfx950).
 //
-// Level 1 (chunk_select_emit, one wave per chunk of 64 x kItems keys): the k smallest keys of the
-// chunk, exactly (threshold from a per-chunk histogram), ties to the lowest index, written as candidates
+// Level 1, one wave per chunk of 64 x kItems keys: the smallest keys of the chunk, exactly (threshold
+// from a per-chunk histogram in LDS), ties to the lowest index, written as candidates
 //     (key << 48) | (offset inside the chunk << 32) | 32-bit payload
-// in (below threshold, tied) x ascending-index order, plus a 512-bin byte histogram of their keys.
-// Level 2 (final_select, one workgroup of 512 threads per row): sums the chunk histograms; the prefix
-// sum gives the global threshold and the tie quota without any search (the k smallest keys of a row
-// are always among the per-chunk winners).  Chunks are concatenated in index order and every list
-// keeps its order, so "ties to the lowest index" carries over: the selected candidates are emitted in
-// that order, ranks from DPP prefix scans, no atomics.
+// in (below threshold, tied) x ascending-index order.  Two forms:
+//   chunk_select_capped  a short list of kc entries (16 for a long row): a chunk holds k / chunks of
+//                        the selection on average.  The list is a prefix of the chunk in (key, index)
+//                        order, so the second level can tell from its last entry whether the chunk
+//                        may hold more of the selection than the list, and then goes back to the
+//                        chunk's keys (fused_step.hip: select_attend_kernel; topk.hip:
+//                        select_final_capped_kernel).  wave_plan_from_hist reads threshold and tie
+//                        quota off a 512-bin histogram, for both levels.
+//   chunk_select_emit    a list of the full k plus a 512-bin byte histogram of its keys; the second
+//                        level (final_select, one workgroup of 512 threads per row) sums the chunk
+//                        histograms and needs no way back to the keys (topk.hip, rows beyond 131072
+//                        keys).
+// Chunks are concatenated in index order and every list keeps its order, so "ties to the lowest
+// index" carries over: the selected candidates are ranked by DPP prefix scans, no atomics.
 #pragma once
 
 #include "select.h"
