@@ -244,3 +244,56 @@ def test_ops_reject_cpu_tensors():
         U.append_kvh(x, x, x, c, 0)
     with pytest.raises(RuntimeError):
         U.hadamard_transform(x)
+
+
+def test_step_plan_covers_every_sequence_with_balanced_chunks():
+    """The geometry the two-launch step derives from the sizes of a call (adamas_step_plan): the
+    chunks tile the past tokens of the longest sequence in 16-token units, differ by at most one
+    unit for a single sequence, fit the workgroup (at most four passes of 512 tokens) and the
+    second launch (at most 64 chunks, 1024 candidate slots per head for one sequence, 2048 for a
+    batch; a power of two of 8 .. 256 slots per chunk, never more than the budget needs)."""
+    lens = sorted(set([2, 3, 17, 18, 33, 511, 512, 513, 514, 1000, 4096, 4097, 8192, 8193, 16384, 16385,
+                       16400, 20000, 32767, 32768, 32769, 32784, 32785, 33024, 36864, 40000, 65536, 65537,
+                       100000, 131056, 131072] + list(range(2, 140000, 3571))))
+    for batch in (1, 2, 16):
+        for heads in (32, 64):
+            for budget in (2, 16, 64, 128, 200, 256):
+                for L in lens:
+                    p = _lib.step_plan(batch, heads, L, budget)
+                    where = (batch, heads, L, budget, p)
+                    if not p["ok"]:
+                        assert L - 1 > 64 * 2048 or (batch > 1 and L - 1 > 64 * 2048), where
+                        continue
+                    units = (L - 1 + 15) // 16
+                    assert 1 <= p["chunks"] <= 64, where
+                    assert p["heads"] in (4, 8) and heads % p["heads"] == 0, where
+                    # the chunks cover all units: a single sequence is tiled exactly, a batch is
+                    # covered by fixed-size chunks
+                    total = p["chunks"] * p["units_q"] + p["units_r"]
+                    if batch == 1 and p["units_r"] == 0 and p["units_q"] % 32 == 0 and p["chunks"] * p["units_q"] > units:
+                        assert total - units < p["units_q"], where      # fixed 512-token chunks
+                    elif batch == 1:
+                        assert total == units or total - units < p["units_q"], where
+                    else:
+                        assert total >= units and p["units_r"] == 0, where
+                    assert p["units_r"] < p["chunks"], where
+                    longest = p["units_q"] + (1 if p["units_r"] else 0)
+                    assert 1 <= p["passes"] <= 4 and longest <= 32 * p["passes"], where
+                    assert longest > 32 * (p["passes"] - 1), where
+                    assert p["partial"] == int(p["units_r"] != 0 or p["units_q"] % 32 != 0), where
+                    kc = p["kc"]
+                    assert kc in (8, 16, 32, 64, 128, 256), where
+                    assert p["chunks"] * kc <= (1024 if batch == 1 else 2048) or kc == 8, where
+                    # never more slots than the budget can use (rounded up to a power of two, at least 8)
+                    need = 8
+                    while need < budget - 1:
+                        need *= 2
+                    assert kc <= need, where
+    # what the headline workloads get
+    assert _lib.step_plan(1, 32, 32768, 128) == {"ok": 1, "heads": 8, "chunks": 64, "units_q": 32, "units_r": 0,
+                                                 "passes": 1, "partial": 0, "kc": 16}
+    p = _lib.step_plan(1, 32, 33024, 128)
+    assert (p["chunks"], p["units_q"], p["units_r"], p["passes"], p["partial"]) == (64, 32, 16, 2, 1)
+    assert _lib.step_plan(1, 32, 131072, 256)["passes"] == 4
+    assert _lib.step_plan(16, 32, 32768, 128)["kc"] == 32
+    assert _lib.step_plan(1, 32, 32768, 1024)["ok"] == 0       # budgets above 256 take the histogram path

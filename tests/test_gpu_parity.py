@@ -935,6 +935,26 @@ def test_paging_identity_vs_shuffled(gpu_device):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("scale", SCALES)
+def test_step_gives_the_same_bits_every_time(gpu_device, scale):
+    """The two-launch step on changing queries, each repeated: outputs and selections must agree with
+    themselves bit for bit (ranks come from prefix scans, nothing is decided by arrival order), also
+    where chunks are scored again (the orthonormal scale gives long runs of equal distances)."""
+    L, budget = 33000, 128
+    seq = _device_sequence(gpu_device, L, 5)
+    ctrl = T.make_controller(gpu_device, L, budget, 16, shuffle_seed=9, scale=scale)
+    T.fill_sequence(ctrl, seq.k[:L - 1], seq.v[:L - 1])
+    T.decode_append(ctrl, seq.q[None], seq.k[L - 1:], seq.v[L - 1:])
+    g = torch.Generator(device=gpu_device).manual_seed(11)
+    for it in range(100):
+        q = (torch.randn(1, 32, 128, generator=g, device=gpu_device) * (1 + it % 4)).half()
+        q_code = U.pack_2bit(U.hadamard_transform(q, scale=ctrl.hadamard_scale))
+        a, sa = U.decode_step(q, q_code, ctrl, 0, return_indices=True)
+        a, sa = a.clone(), sa.clone()
+        b, sb = U.decode_step(q, q_code, ctrl, 0, return_indices=True)
+        assert torch.equal(a, b) and torch.equal(sa, sb), it
+
+
 def test_split_merge_inside_the_launch_gives_the_same_bits_every_time(gpu_device):
     """The attention over 1023 rows per head is cut into eight splits whose partial results are
     merged by the last workgroup to arrive, inside the launch (write-through stores, an arrival
