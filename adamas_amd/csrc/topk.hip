@@ -69,30 +69,8 @@ __device__ __forceinline__ uint32_t row_length(const SelectArgs& a, uint32_t row
 }
 
 // keys of items e0..e0+7 of a row of values (n = row length)
-// kPadded: the row is backed up to a multiple of 8 elements (and vec_ok holds), so the group that
-// holds the end of the row is read with one 128-bit load as well and masked afterwards.
-template <bool kPadded = false>
 __device__ __forceinline__ void load_value_keys(const uint16_t* vrow, uint32_t e0, uint32_t n,
                                                 bool vec_ok, uint32_t key_mode, uint32_t* keys) {
-  if (kPadded) {
-    if (e0 < n) {
-      const uint4 v = *reinterpret_cast<const uint4*>(vrow + e0);
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        keys[2 * i] = make_key(w[i] & 0xffffu, key_mode);
-        keys[2 * i + 1] = make_key(w[i] >> 16, key_mode);
-      }
-      if (e0 + 8 > n) {
-#pragma unroll
-        for (int r = 0; r < 8; ++r) keys[r] = (e0 + r < n) ? keys[r] : kInvalidKey;
-      }
-    } else {
-#pragma unroll
-      for (int r = 0; r < 8; ++r) keys[r] = kInvalidKey;
-    }
-    return;
-  }
   if (vec_ok && e0 + 8 <= n) {
     const uint4 v = *reinterpret_cast<const uint4*>(vrow + e0);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -871,8 +849,8 @@ struct HistEmitShared {
 // kKeyMode >= 0: the key format is known at compile time and the rows are read with 128-bit loads
 // (the caller has checked their alignment); -1: both are taken from the arguments.  The instances
 // with a fixed format leave out the element-wise loads and the other formats' conversions, which
-// are most of the code of the general one.  kPadded: see load_value_keys.
-template <int kKeyMode, bool kPadded = false>
+// are most of the code of the general one.
+template <int kKeyMode>
 __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
     SelectArgs a, const uint16_t* __restrict__ hist, uint32_t n_chunks, uint32_t chunks_per_slab) {
   const uint32_t key_mode = kKeyMode >= 0 ? static_cast<uint32_t>(kKeyMode) : a.key_mode;
@@ -897,7 +875,7 @@ __global__ __launch_bounds__(kEmitThreads) void select_hist_emit_kernel(
   uint32_t keys[kEmitItems];
 #pragma unroll
   for (int j = 0; j < kEmitItems / 8; ++j)
-    load_value_keys<kPadded>(vrow, e0 + j * 8, n, vec_ok, key_mode, &keys[j * 8]);
+    load_value_keys(vrow, e0 + j * 8, n, vec_ok, key_mode, &keys[j * 8]);
 
   // ---- chunk rows: thread (part, seg) adds bins 8*seg .. 8*seg+7 of rows part, part + 4, ...
   {
