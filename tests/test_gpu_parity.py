@@ -678,6 +678,43 @@ def test_step_large_budget_ragged_batch(gpu_device):
         assert np.abs(T.np16(o_f)[b].astype(np.float64) - ora["out"]).max() <= ATTN_TOL
 
 
+@pytest.mark.parametrize("scale", SCALES)
+def test_step_short_sequences_in_a_long_batch(gpu_device, scale):
+    """A batch whose longest sequence fixes 64 chunks and lists of 32 entries, next to sequences
+    shorter than the budget, shorter than a list, and between the two: a short sequence has all its
+    tokens in chunk 0, whose list then runs out although the whole sequence is selected."""
+    lens = [32000, 100, 40, 600, 33, 129, 8000, 2]
+    budget = 128
+    assert _lib.step_plan(len(lens), 32, max(lens), budget)["kc"] == 32
+    g = torch.Generator().manual_seed(21)
+    seqs = [synth.make_sequence(L, 4, g) for L in lens]
+    B = len(lens)
+    ctrl = T.make_controller(gpu_device, max(lens), budget, 16, batch_size=B, shuffle_seed=6, scale=scale)
+    for b, s in enumerate(seqs):
+        if lens[b] > 1:
+            T.fill_sequence(ctrl, s.k[:-1].to(gpu_device), s.v[:-1].to(gpu_device), seq_idx=b)
+    q = torch.stack([s.q for s in seqs]).to(gpu_device)
+    kn = torch.stack([s.k[-1] for s in seqs]).to(gpu_device)
+    vn = torch.stack([s.v[-1] for s in seqs]).to(gpu_device)
+    q_code = T.decode_append(ctrl, q, kn, vn)
+    est = U.decode_estimate(q_code, ctrl, 0)
+    U.decode_topk(est, ctrl)
+    sel = ctrl.topk_dindices_buffer.clone()
+    o = U.decode_sparse_attn(q, ctrl, 0, sel)
+    o_f, sel_f = U.decode_step(q, q_code, ctrl, 0, return_indices=True)
+    a = np.sort(T.np16(sel).astype(np.int64), axis=1)
+    b_ = np.sort(T.np16(sel_f).astype(np.int64), axis=1)
+    assert np.array_equal(a, b_)
+    assert np.abs(T.np16(o).astype(np.float64) - T.np16(o_f).astype(np.float64)).max() <= ATTN_TOL
+    for b, s in enumerate(seqs):
+        if lens[b] > 700:
+            continue
+        ora = T.oracle_step(s.q, s.k, s.v, budget, scale=scale)
+        ok, h = T.sets_equal(T.np16(sel_f[b * 32:(b + 1) * 32]), ora["sets"], lens[b])
+        assert ok, (b, h)
+        assert np.abs(T.np16(o_f)[b].astype(np.float64) - ora["out"]).max() <= ATTN_TOL, b
+
+
 def test_step_wide_distance_spread(gpu_device):
     """Two past tokens equal the query (distance 0) while every other token has saturated codes
     (distances around 190): the k-th nearest lies far above the minimum of its chunk, and the
