@@ -39,7 +39,11 @@ __global__ __launch_bounds__(256) void estimate_kernel(
   const uint32_t t0 = (blockIdx.x * 4u + static_cast<uint32_t>(wave_id_uniform())) * kTokPerWave;
   if (n <= 0 || t0 >= static_cast<uint32_t>(n)) return;
 
-  const uint32_t head = seg * 32u + (static_cast<uint32_t>(lane) >> 1);
+  // (a head count that is no multiple of 32 leaves lanes of the last group without a head: they
+  // compute the last head's distances again and store nothing)
+  const uint32_t head_lane = seg * 32u + (static_cast<uint32_t>(lane) >> 1);
+  const bool head_ok = head_lane < num_heads;
+  const uint32_t head = head_ok ? head_lane : num_heads - 1u;
   const uint32_t half = static_cast<uint32_t>(lane) & 1u;
   const uint4 qraw = *reinterpret_cast<const uint4*>(
       q_code + (static_cast<size_t>(b) * num_heads + head) * kCodeWords + half * 8u);
@@ -93,6 +97,7 @@ __global__ __launch_bounds__(256) void estimate_kernel(
   }
   const uint32_t ts = t0 + half * 8u;
   uint16_t* dst = out + static_cast<int64_t>(b) * out_bs + static_cast<int64_t>(head) * out_hs + ts;
+  if (!head_ok) return;
   if (vec_ok && ts + 8u <= static_cast<uint32_t>(n)) {
     *reinterpret_cast<uint4*>(dst) = make_uint4(w0, w1, w2, w3);
   } else {
@@ -151,7 +156,7 @@ extern "C" int adamas_estimate(const void* q_code, const void* code_data,
   if (!q_code || !code_data || !page_indices || !page_indptr || !seq_lens || !out || batch == 0 ||
       page_size == 0)
     return ADAMAS_E_BADARG;
-  if (num_heads == 0 || num_heads % 32 != 0) return ADAMAS_E_UNSUPPORTED;
+  if (num_heads == 0) return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
   // the kernel takes head / group from a 16-bit reciprocal (kv_head_of)
   if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;
@@ -166,7 +171,7 @@ extern "C" int adamas_estimate(const void* q_code, const void* code_data,
                            out_head_stride % 8 == 0 && out_batch_stride % 8 == 0)
                               ? 1u
                               : 0u;
-  dim3 grid((n_max + kTokPerBlock - 1) / kTokPerBlock, batch, num_heads / 32);
+  dim3 grid((n_max + kTokPerBlock - 1) / kTokPerBlock, batch, (num_heads + 31) / 32);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define ADAMAS_LAUNCH_ESTIMATE(PG)                                                              \
   hipLaunchKernelGGL(estimate_kernel<PG>, grid, dim3(256), 0, s,                                \

@@ -1104,7 +1104,7 @@ static bool fused_eligible(const WorkspaceLayout& w) { return w.plan.ok != 0; }
 
 extern "C" int adamas_step_fused_supported(uint32_t batch, uint32_t num_heads,
                                            uint32_t max_seq_len, uint32_t budget) {
-  if (batch == 0 || num_heads == 0 || num_heads % 32 != 0 || budget == 0 || max_seq_len == 0)
+  if (batch == 0 || num_heads == 0 || num_heads % 8 != 0 || budget == 0 || max_seq_len == 0)
     return 0;
   return fused_eligible(workspace_layout(batch, num_heads, max_seq_len, budget)) ? 1 : 0;
 }
@@ -1112,7 +1112,7 @@ extern "C" int adamas_step_fused_supported(uint32_t batch, uint32_t num_heads,
 extern "C" int adamas_step_plan(uint32_t batch, uint32_t num_heads, uint32_t max_seq_len,
                                 uint32_t budget, uint32_t* plan_out) {
   if (!plan_out) return ADAMAS_E_BADARG;
-  const StepPlan p = (batch && num_heads && num_heads % 32 == 0)
+  const StepPlan p = (batch && num_heads && num_heads % 8 == 0)
                          ? step_plan(batch, num_heads, max_seq_len, budget)
                          : StepPlan{};
   const uint32_t v[8] = {p.ok, p.heads, p.chunks, p.units_q, p.units_r, p.passes, p.partial, p.kc};
@@ -1148,7 +1148,7 @@ static int step_candidates_impl(const void* q_code, const void* code_data,
       !seq_lens || !workspace ||
       budget == 0 || max_seq_len == 0 || batch == 0 || page_size == 0)
     return ADAMAS_E_BADARG;
-  if (num_heads == 0 || num_heads % 32 != 0 || batch > 65535) return ADAMAS_E_UNSUPPORTED;
+  if (num_heads == 0 || num_heads % 8 != 0 || batch > 65535) return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
   // the kernels take head / group from a 16-bit reciprocal (kv_head_of)
   if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;
@@ -1261,7 +1261,7 @@ static int step_attend_impl(const void* q, void* kv_data, void* code_data,
       !seq_lens || !out || !workspace ||
       budget == 0 || max_seq_len == 0 || batch == 0 || page_size == 0)
     return ADAMAS_E_BADARG;
-  if (head_dim != kHeadDim || num_heads == 0 || num_heads % 32 != 0 || batch > 65535)
+  if (head_dim != kHeadDim || num_heads == 0 || num_heads % 8 != 0 || batch > 65535)
     return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
   // the kernels take head / group from a 16-bit reciprocal (kv_head_of)
@@ -1359,7 +1359,7 @@ extern "C" int adamas_decode_step_f(const void* q, const void* q_code, const voi
   if (!q || !q_code || !kv_data || !code_data || !page_indices || !page_indptr || !seq_lens ||
       !out || !workspace || budget == 0 || max_seq_len == 0 || batch == 0 || page_size == 0)
     return ADAMAS_E_BADARG;
-  if (head_dim != kHeadDim || num_heads == 0 || num_heads % 32 != 0) return ADAMAS_E_UNSUPPORTED;
+  if (head_dim != kHeadDim || num_heads == 0 || num_heads % 8 != 0) return ADAMAS_E_UNSUPPORTED;
   if (num_kv_heads == 0 || num_heads % num_kv_heads != 0) return ADAMAS_E_UNSUPPORTED;
   // the kernels take head / group from a 16-bit reciprocal (kv_head_of)
   if (static_cast<uint64_t>(num_heads) * (num_heads / num_kv_heads) >= 65536u) return ADAMAS_E_UNSUPPORTED;

@@ -55,8 +55,8 @@ class InferenceController:
                 f"Adamas HIP path supports torch.float16 and torch.bfloat16 only, got {dtype}")
         if head_dim != 128:
             raise RuntimeError("Adamas HIP path supports head_dim 128 only")
-        if num_heads % 32 != 0:
-            raise RuntimeError("Adamas HIP path needs num_heads to be a multiple of 32")
+        if num_heads % 8 != 0:
+            raise RuntimeError("Adamas HIP path needs num_heads to be a multiple of 8")
         self.device = torch.device(device)
         self.dtype = dtype
         self.num_layers = num_layers

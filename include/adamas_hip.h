@@ -46,7 +46,7 @@ typedef void* adamas_stream_t;
 
 /* Negative error codes (positive values are hipError_t). */
 #define ADAMAS_E_BADARG (-1)      /* null pointer, zero size, inconsistent sizes          */
-#define ADAMAS_E_UNSUPPORTED (-2) /* head_dim != 128, num_heads not a multiple of 32, ... */
+#define ADAMAS_E_UNSUPPORTED (-2) /* head_dim != 128, num_heads not a multiple of 8, ... */
 #define ADAMAS_E_WORKSPACE (-3)   /* workspace too small                                  */
 #define ADAMAS_E_ALIGN (-4)       /* pointer or stride not aligned as documented          */
 #define ADAMAS_E_SCRATCH (-5)     /* sizes beyond the static scratch of adamas_decode_step_noalloc */

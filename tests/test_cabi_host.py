@@ -71,7 +71,7 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.adamas_append_decode(*([None] * 10), 1, 32, 32, 128, 16, 1.0, 0, None) == -1
     assert lib.adamas_append_prefill(16, 16, None, 4, 0, 16, 16, 16, 1, 32, 64, 16, 1.0, 0, None) == -2
     assert lib.adamas_append_prefill(16, 16, None, 40, 0, 16, 16, 16, 1, 32, 128, 16, 1.0, 0, None) == -1
-    assert lib.adamas_estimate(16, 16, 16, 16, 16, 16, 8, 8, 0, 1, 24, 24, 16, 100, None) == -2   # heads % 32
+    assert lib.adamas_estimate(16, 16, 16, 16, 16, 16, 8, 8, 0, 1, 0, 24, 16, 100, None) == -2    # no heads
     assert lib.adamas_estimate(16, 16, 16, 16, 16, 16, 8, 8, 0, 1, 32, 5, 16, 100, None) == -2    # 32 % kv heads
     assert lib.adamas_estimate(16, 16, 16, 16, 16, 16, 8, 8, 7, 1, 32, 32, 16, 100, None) == -1   # format
     assert lib.adamas_estimate(16, 16, 16, 16, 16, 16, 8, 8, 0, 1, 32, 8, 16, 1, None) == 0      # nothing to do
@@ -94,6 +94,8 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.adamas_step_fused_supported(1, 32, 131072, 256) == 1       # 64 chunks of 2048 tokens
     assert lib.adamas_step_fused_supported(1, 32, 262144, 256) == 0       # too many candidate slots
     assert lib.adamas_step_fused_supported(1, 32, 4096, 1024) == 0        # budget beyond 256
+    assert lib.adamas_step_fused_supported(1, 40, 32768, 128) == 1        # any multiple of 8 heads
+    assert lib.adamas_step_fused_supported(1, 36, 32768, 128) == 0
     assert lib.adamas_step_candidates(16, 16, 16, 16, 16, 1024, 256, 1 << 30, 1, 32, 32, 16, 4096, 0, None) == -2
     assert lib.adamas_step_candidates(16, 16, 16, None, 16, 128, 256, 1 << 30, 1, 32, 32, 16, 4096, 0, None) == -1
     assert lib.adamas_step_attend(16, 16, 16, 16, 16, 16, 128, 16, None, None, 0, 1, 32, 32, 128, 16, 0.1, 4096, 0, None) == -1
@@ -256,7 +258,7 @@ def test_step_plan_covers_every_sequence_with_balanced_chunks():
                        16400, 20000, 32767, 32768, 32769, 32784, 32785, 33024, 36864, 40000, 65536, 65537,
                        100000, 131056, 131072] + list(range(2, 140000, 3571))))
     for batch in (1, 2, 16):
-        for heads in (32, 64):
+        for heads in (32, 40, 64):
             for budget in (2, 16, 64, 128, 200, 256):
                 for L in lens:
                     p = _lib.step_plan(batch, heads, L, budget)

@@ -382,9 +382,11 @@ def test_gemv_silu_gate_equals_gemv_then_silu_mul(gpu_device, inter, k):
     assert torch.equal(U.gemv_silu_gate(w, x), U.silu_mul(U.gemv(w, x)))
 
 
-def test_sixty_four_heads(gpu_device):
-    """Every kernel takes any multiple of 32 heads; the other tests use 32."""
-    cfg = DecoderConfig(num_layers=2, hidden=8192, num_heads=64, head_dim=128, intermediate=256,
+@pytest.mark.parametrize("heads", [64, 40])
+def test_other_head_counts(gpu_device, heads):
+    """Every kernel takes any multiple of 8 heads (40: the 13B shape of the model family); the other
+    tests use 32."""
+    cfg = DecoderConfig(num_layers=2, hidden=128 * heads, num_heads=heads, head_dim=128, intermediate=256,
                         vocab=256, dense_layers=1)
     m = LlamaShapedDecoder(cfg, gpu_device, seed=6)
     ids = torch.randint(0, cfg.vocab, (200,), generator=torch.Generator().manual_seed(2)).to(gpu_device)

@@ -912,7 +912,9 @@ def test_empty_and_single_token_sequences_through_the_c_abi(gpu_device):
 
 @pytest.mark.parametrize("hq,hkv,page_size,budget", [
     (32, 8, 16, 96), (64, 16, 16, 96), (32, 32, 16, 96), (32, 4, 3, 96), (32, 16, 16, 96),
-    (64, 8, 7, 96), (32, 8, 16, 400), (64, 16, 5, 1000)])
+    (64, 8, 7, 96), (32, 8, 16, 400), (64, 16, 5, 1000),
+    # head counts that are no multiple of 32 (40 heads: the 13B shape of the model family)
+    (40, 40, 16, 96), (40, 8, 16, 96), (40, 10, 7, 400), (8, 8, 16, 64), (24, 8, 16, 96), (40, 40, 16, 1000)])
 @pytest.mark.parametrize("fused_append", [True, False])
 @pytest.mark.parametrize("scale", SCALES)
 def test_grouped_query_attention_step(gpu_device, hq, hkv, page_size, budget, fused_append, scale):
