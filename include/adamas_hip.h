@@ -247,7 +247,8 @@ int adamas_sparse_decode_f(const void* q, const void* kv_data, const int32_t* pa
  * estimate -> select (budget-1 nearest past tokens, ties to the lowest index) -> attention over the
  * selection plus the current token.  Sequences with seq_lens[b] <= budget attend to everything.
  * q_code comes from adamas_append_decode.  sel_out (optional) [batch*num_heads][budget-1] int32
- * receives the selected logical positions.
+ * receives the selected logical positions (a set: the order within a row is deterministic but not
+ * specified; unused entries are -1).
  * page_table_stride: 0 = sequence b's page list starts at page_indices[page_indptr[b]]; otherwise it
  * starts at page_indices[b * page_table_stride] (fixed-stride tables), every entry of a row must be
  * a valid page id, and the kernels fetch page ids and sequence length side by side instead of one
